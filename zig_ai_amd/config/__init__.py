@@ -1,7 +1,7 @@
 """Configurations and the one registry from an architecture's name to its model.
 
-An entry couples the name that config.json carries in ``architectures[0]`` with
-a typed configuration class.  The class parses config.json (``from_dict``),
+An entry couples the name that config.json carries in ``architectures[0]`` (or as
+the string ``architecture``) with a typed configuration class.  The class parses config.json (``from_dict``),
 writes it back (``to_dict``) and describes the model as parts (``to_spec``);
 the generic decoder is assembled from that description, so registering a
 configuration class registers the model.
@@ -15,6 +15,7 @@ from typing import Any, Callable, Dict, Mapping
 
 from .spec import ConfigError, LayerCall, LayerSpec, ModelSpec, PartSpec  # noqa: F401
 from .lfm2 import Lfm2Config, feed_forward_width  # noqa: F401
+from .rudilix import RudilixConfig  # noqa: F401
 
 _ARCHITECTURES: Dict[str, Any] = {}
 
@@ -33,6 +34,8 @@ def known_architectures() -> list:
 
 def config_from_dict(data: Mapping[str, Any]):
     archs = data.get("architectures")
+    if not archs and isinstance(data.get("architecture"), str):
+        archs = [data["architecture"]]
     if not archs or not isinstance(archs, (list, tuple)) or not isinstance(archs[0], str):
         raise ConfigError(
             "config.json has no architectures entry; known architectures: "
@@ -62,3 +65,4 @@ def load_config(model_dir: str):
 
 
 register_architecture("Lfm2ForCausalLM", Lfm2Config)
+register_architecture("Rudilix", RudilixConfig)

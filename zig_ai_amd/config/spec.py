@@ -46,6 +46,9 @@ class LayerSpec:
 
     parts: Mapping[str, PartSpec]
     arrangement: str = "pre_norm_residual"
+    # constants of the arrangement itself (how much of each part enters the stream, say);
+    # handed to its constructor as keywords
+    params: Mapping[str, Any] = field(default_factory=dict)
 
     @classmethod
     def pre_norm(cls, mixer: PartSpec, feed_forward: PartSpec, mixer_norm: PartSpec,

@@ -120,3 +120,41 @@ extern "C" int za_copy_columns(const void* in, int in_dtype, int in_width, int c
 #undef ZA_COPY_COLUMNS
   return za_launch_status();
 }
+
+// A gated linear unit with bounded inputs, on the fused gate|up projection:
+//   g = min(gu[t, i], limit);  u = clamp(gu[t, I + i], -limit, limit)
+//   out[t, i] = g * sigmoid(alpha * g) * (u + up_offset)
+// in 32-bit.  `limit <= 0` means no bound.
+template <typename T>
+__global__ void __launch_bounds__(256)
+clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ out, int n_tokens, int inter,
+                   float limit, float alpha, float up_offset) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t total = (size_t)n_tokens * inter;
+  if (idx >= total) return;
+  const size_t t = idx / inter, i = idx % inter;
+  float g = to_f32<T>(gu[t * 2 * inter + i]);
+  float u = to_f32<T>(gu[t * 2 * inter + inter + i]);
+  if (limit > 0.f) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+  }
+  out[idx] = from_f32<T>(g * (1.0f / (1.0f + expf(-alpha * g))) * (u + up_offset));
+}
+
+extern "C" int za_clamped_glu(const void* gu, void* out, int dtype, int n_tokens, int inter,
+                              float limit, float alpha, float up_offset, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  if (n_tokens < 0 || inter <= 0 || !gu || !out) return ZA_ERR_ARG;
+  const size_t total = (size_t)n_tokens * inter;
+  dim3 grid((unsigned)((total + 255) / 256)), block(256);
+  if (dtype == 0)
+    hipLaunchKernelGGL((clamped_glu_kernel<float>), grid, block, 0, stream, (const float*)gu,
+                       (float*)out, n_tokens, inter, limit, alpha, up_offset);
+  else if (dtype == 1)
+    hipLaunchKernelGGL((clamped_glu_kernel<bf16_t>), grid, block, 0, stream, (const bf16_t*)gu,
+                       (bf16_t*)out, n_tokens, inter, limit, alpha, up_offset);
+  else
+    return ZA_ERR_UNSUPPORTED;
+  return za_launch_status();
+}

@@ -43,12 +43,19 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
                        const int* __restrict__ wi_row0, const int* __restrict__ wi_count,
                        float* __restrict__ part_acc, float* __restrict__ part_ml, int nh, int nkv,
                        int d, int page_size, float scale, int window, int keys_per_split,
-                       int nsplit) {
+                       int nsplit, int dv, const T* __restrict__ gate, int gate_stride,
+                       int gate_col, float out_scale) {
+  // `dv`: width of a value (keys and queries have `d`); a page holds the keys of all
+  // heads, [kv_head][offset][d], then the values turned round, [kv_head][dv][offset].
+  // `gate`: when given, head h of token t is multiplied by
+  // sigmoid(gate[t * gate_stride + gate_col + h]) * out_scale.
   extern __shared__ float smem[];
-  const int ldk = d + 1;
+  const int ldk = d + 1, ldv = dv + 1;
+  const size_t page_elems = (size_t)nkv * page_size * (d + dv);
+  const size_t value_base = (size_t)nkv * page_size * d;
   float* Ks = smem;                       // [KT][d + 1]
-  float* Vs = Ks + KT * ldk;              // [KT][d + 1]
-  float* Qs = Vs + KT * ldk;              // [AT_MAX_ROWS][d]
+  float* Vs = Ks + KT * ldk;              // [KT][dv + 1]
+  float* Qs = Vs + KT * ldv;              // [AT_MAX_ROWS][d]
   float* Ps = Qs + AT_MAX_ROWS * d;       // [AT_WAVES][64]
 
   const int item = blockIdx.x, g = blockIdx.y, z = blockIdx.z;
@@ -102,7 +109,7 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
         ok = page >= 0;
       }
       if (ok) {
-        load8<T>(kv + ((((size_t)page * 2) * nkv + g) * page_size + kp % page_size) * d + c, kx);
+        load8<T>(kv + page * page_elems + ((size_t)g * page_size + kp % page_size) * d + c, kx);
       } else {
 #pragma unroll
         for (int i = 0; i < 8; ++i) kx[i] = 0.f;
@@ -119,10 +126,10 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
       if (kp >= lo && kp <= range_hi) {
         const int page = table[kp / page_size];
         if (page >= 0)
-          vsrc = kv + (((size_t)page * 2 + 1) * nkv + g) * page_size * d + kp % page_size;
+          vsrc = kv + page * page_elems + value_base + (size_t)g * dv * page_size + kp % page_size;
       }
-      for (int dd = tid / KT; dd < d; dd += 256 / KT)
-        Vs[j * ldk + dd] = vsrc ? to_f32<T>(vsrc[(size_t)dd * page_size]) : 0.f;
+      for (int dd = tid / KT; dd < dv; dd += 256 / KT)
+        Vs[j * ldv + dd] = vsrc ? to_f32<T>(vsrc[(size_t)dd * page_size]) : 0.f;
     }
     __syncthreads();
 
@@ -155,11 +162,11 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
 #pragma unroll
           for (int c = 0; c < AT_DPL; ++c) {
             const int dd = lane + 64 * c;
-            if (64 * c < d) {
+            if (64 * c < dv) {
               float a = acc[lr][c] * alpha;
-              if (dd < d) {
+              if (dd < dv) {
 #pragma unroll 8
-                for (int j = 0; j < KT; ++j) a = fmaf(Ps[wave * 64 + j], Vs[j * ldk + dd], a);
+                for (int j = 0; j < KT; ++j) a = fmaf(Ps[wave * 64 + j], Vs[j * ldv + dd], a);
               }
               acc[lr][c] = a;
             }
@@ -177,19 +184,24 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
       const int tok = row0 + r / G, h = g * G + r % G;
       if (nsplit == 1) {
         const float inv = l[lr] > 0.f ? 1.0f / l[lr] : 0.f;
-        T* o = out + ((size_t)tok * nh + h) * d;
+        float mult = 1.0f;
+        if (gate) {
+          const float gl = to_f32<T>(gate[(size_t)tok * gate_stride + gate_col + h]);
+          mult = out_scale / (1.0f + expf(-gl));
+        }
+        T* o = out + ((size_t)tok * nh + h) * dv;
 #pragma unroll
         for (int c = 0; c < AT_DPL; ++c) {
           const int dd = lane + 64 * c;
-          if (dd < d) o[dd] = from_f32<T>(acc[lr][c] * inv);
+          if (dd < dv) o[dd] = from_f32<T>(gate ? acc[lr][c] * inv * mult : acc[lr][c] * inv);
         }
       } else {
         const size_t pidx = ((size_t)tok * nh + h) * nsplit + z;
-        float* pa = part_acc + pidx * d;
+        float* pa = part_acc + pidx * dv;
 #pragma unroll
         for (int c = 0; c < AT_DPL; ++c) {
           const int dd = lane + 64 * c;
-          if (dd < d) pa[dd] = acc[lr][c];
+          if (dd < dv) pa[dd] = acc[lr][c];
         }
         if (lane == 0) {
           part_ml[pidx * 2] = m[lr];
@@ -1049,9 +1061,10 @@ static int launch_attention(const void* q, void* out, const void* kv, const int*
                             int bt_stride, const int* positions, const int* wi_seq,
                             const int* wi_row0, const int* wi_count, int n_items, float* part_acc,
                             float* part_ml, int nh, int nkv, int d, int page_size, float scale,
-                            int window, int keys_per_split, int nsplit, hipStream_t stream) {
-  const size_t shmem =
-      ((size_t)2 * KT * (d + 1) + (size_t)AT_MAX_ROWS * d + AT_WAVES * 64) * sizeof(float);
+                            int window, int keys_per_split, int nsplit, int dv, const void* gate,
+                            int gate_stride, int gate_col, float out_scale, hipStream_t stream) {
+  const size_t shmem = ((size_t)KT * (d + 1) + (size_t)KT * (dv + 1) + (size_t)AT_MAX_ROWS * d +
+                        AT_WAVES * 64) * sizeof(float);
   auto kernel = paged_attention_kernel<T, KT>;
   static size_t allowed = 0;
   if (shmem > allowed) {
@@ -1063,9 +1076,53 @@ static int launch_attention(const void* q, void* out, const void* kv, const int*
   dim3 grid(n_items, nkv, nsplit), block(256);
   hipLaunchKernelGGL(kernel, grid, block, shmem, stream, (const T*)q, (T*)out, (const T*)kv,
                      block_table, bt_stride, positions, wi_seq, wi_row0, wi_count, part_acc,
-                     part_ml, nh, nkv, d, page_size, scale, window, keys_per_split, nsplit);
+                     part_ml, nh, nkv, d, page_size, scale, window, keys_per_split, nsplit, dv,
+                     (const T*)gate, gate_stride, gate_col, out_scale);
   return za_launch_status();
 }
+
+// Every head of every token times sigmoid(gate[t * gate_stride + gate_col + h]) * scale:
+// the output gate of an attention whose kernel did not apply it itself.
+template <typename T>
+__global__ void __launch_bounds__(256)
+head_gate_kernel(T* __restrict__ out, const T* __restrict__ gate, int gate_stride, int gate_col,
+                 int nh, int dv, float out_scale, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t row = idx / dv;             // token * nh + head
+  const size_t tok = row / nh;
+  const int h = (int)(row % nh);
+  const float gl = to_f32<T>(gate[tok * gate_stride + gate_col + h]);
+  out[idx] = from_f32<T>(to_f32<T>(out[idx]) * (out_scale / (1.0f + expf(-gl))));
+}
+
+extern "C" int za_head_gate(void* out, const void* gate, int dtype, int gate_stride, int gate_col,
+                            int n_tokens, int nh, int dv, float out_scale, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  if (n_tokens < 0 || nh <= 0 || dv <= 0 || !out || !gate || gate_col < 0 ||
+      gate_col + nh > gate_stride)
+    return ZA_ERR_ARG;
+  const size_t total = (size_t)n_tokens * nh * dv;
+  dim3 grid((unsigned)((total + 255) / 256)), block(256);
+  if (dtype == 0)
+    hipLaunchKernelGGL((head_gate_kernel<float>), grid, block, 0, stream, (float*)out,
+                       (const float*)gate, gate_stride, gate_col, nh, dv, out_scale, total);
+  else if (dtype == 1)
+    hipLaunchKernelGGL((head_gate_kernel<bf16_t>), grid, block, 0, stream, (bf16_t*)out,
+                       (const bf16_t*)gate, gate_stride, gate_col, nh, dv, out_scale, total);
+  else
+    return ZA_ERR_UNSUPPORTED;
+  return za_launch_status();
+}
+
+static int paged_attention_any(const void* q, void* out, const void* kv, const int* block_table,
+                               int bt_stride, const int* positions, const int* wi_seq,
+                               const int* wi_row0, const int* wi_count, int n_items,
+                               int n_tokens, float* part_acc, float* part_ml, int dtype, int nh,
+                               int nkv, int d, int page_size, float scale, int window,
+                               int keys_per_split, int nsplit, int dv, const void* gate,
+                               int gate_stride, int gate_col, float out_scale,
+                               hipStream_t stream);
 
 // dtype codes: 0 = float32, 1 = bfloat16
 extern "C" int za_paged_attention(const void* q, void* out, const void* kv, const int* block_table,
@@ -1074,6 +1131,39 @@ extern "C" int za_paged_attention(const void* q, void* out, const void* kv, cons
                                   int n_tokens, float* part_acc, float* part_ml, int dtype, int nh,
                                   int nkv, int d, int page_size, float scale, int window,
                                   int keys_per_split, int nsplit, hipStream_t stream) {
+  return paged_attention_any(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0,
+                             wi_count, n_items, n_tokens, part_acc, part_ml, dtype, nh, nkv, d,
+                             page_size, scale, window, keys_per_split, nsplit, d, nullptr, 0, 0,
+                             1.0f, stream);
+}
+
+// The same with values of width `dv` (a page: keys [kv_head][offset][d], then values
+// [kv_head][dv][offset]) and an optional per-head output gate.
+extern "C" int za_paged_attention_gated(const void* q, void* out, const void* kv,
+                                        const int* block_table, int bt_stride,
+                                        const int* positions, const int* wi_seq,
+                                        const int* wi_row0, const int* wi_count, int n_items,
+                                        int n_tokens, float* part_acc, float* part_ml, int dtype,
+                                        int nh, int nkv, int d, int dv, int page_size, float scale,
+                                        int window, int keys_per_split, int nsplit,
+                                        const void* gate, int gate_stride, int gate_col,
+                                        float out_scale, hipStream_t stream) {
+  if (dv <= 0 || dv % 8 != 0 || dv > AT_MAX_D) return ZA_ERR_UNSUPPORTED;
+  if (gate && (gate_col < 0 || gate_col + nh > gate_stride)) return ZA_ERR_ARG;
+  return paged_attention_any(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0,
+                             wi_count, n_items, n_tokens, part_acc, part_ml, dtype, nh, nkv, d,
+                             page_size, scale, window, keys_per_split, nsplit, dv, gate,
+                             gate_stride, gate_col, out_scale, stream);
+}
+
+static int paged_attention_any(const void* q, void* out, const void* kv, const int* block_table,
+                               int bt_stride, const int* positions, const int* wi_seq,
+                               const int* wi_row0, const int* wi_count, int n_items,
+                               int n_tokens, float* part_acc, float* part_ml, int dtype, int nh,
+                               int nkv, int d, int page_size, float scale, int window,
+                               int keys_per_split, int nsplit, int dv, const void* gate,
+                               int gate_stride, int gate_col, float out_scale,
+                               hipStream_t stream) {
   if (n_items == 0 || n_tokens == 0) return 0;
   if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || d <= 0 || page_size <= 0 ||
       bt_stride <= 0 || nsplit < 1 || !q || !out || !kv || !block_table || !positions ||
@@ -1086,11 +1176,13 @@ extern "C" int za_paged_attention(const void* q, void* out, const void* kv, cons
   int rc;
 #define ZA_AT_ARGS                                                                            \
   q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0, wi_count, n_items, part_acc, \
-      part_ml, nh, nkv, d, page_size, scale, window, keys_per_split, nsplit, stream
+      part_ml, nh, nkv, d, page_size, scale, window, keys_per_split, nsplit, dv, gate,         \
+      gate_stride, gate_col, out_scale, stream
+  const bool small = d <= 128 && dv <= 128;
   if (dtype == 0) {
-    rc = d <= 128 ? launch_attention<float, 64>(ZA_AT_ARGS) : launch_attention<float, 32>(ZA_AT_ARGS);
+    rc = small ? launch_attention<float, 64>(ZA_AT_ARGS) : launch_attention<float, 32>(ZA_AT_ARGS);
   } else if (dtype == 1) {
-    rc = d <= 128 ? launch_attention<bf16_t, 64>(ZA_AT_ARGS)
+    rc = small ? launch_attention<bf16_t, 64>(ZA_AT_ARGS)
                   : launch_attention<bf16_t, 32>(ZA_AT_ARGS);
   } else {
     return ZA_ERR_UNSUPPORTED;
@@ -1100,11 +1192,13 @@ extern "C" int za_paged_attention(const void* q, void* out, const void* kv, cons
   dim3 grid((unsigned)((size_t)n_tokens * nh)), block(64);
   if (dtype == 0)
     hipLaunchKernelGGL((attention_combine_kernel<float>), grid, block, 0, stream, part_acc,
-                       part_ml, (float*)out, d, nsplit, 0);
+                       part_ml, (float*)out, dv, nsplit, 0);
   else
     hipLaunchKernelGGL((attention_combine_kernel<bf16_t>), grid, block, 0, stream, part_acc,
-                       part_ml, (bf16_t*)out, d, nsplit, 0);
-  return za_launch_status();
+                       part_ml, (bf16_t*)out, dv, nsplit, 0);
+  rc = za_launch_status();
+  if (rc != 0 || !gate) return rc;
+  return za_head_gate(out, gate, dtype, gate_stride, gate_col, n_tokens, nh, dv, out_scale, stream);
 }
 
 template <int D, int KT>

@@ -223,3 +223,51 @@ extern "C" int za_embed_gather(const int* tokens, const void* table, int table_d
   }
   return za_launch_status();
 }
+
+// A residual stream that takes its blocks' results with weights:
+//   x <- x + sa * a + sb * b      (b may be absent; 32-bit sum, stored)
+//   out = x / sqrt(mean(x^2) + eps) * weight      (when a norm's weight is given)
+// `a` and `b` are in the storage type TD.  One workgroup a row, two passes.
+template <typename TD, typename TO>
+__global__ void __launch_bounds__(256)
+scaled_add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ a, float sa,
+                          const TD* __restrict__ b, float sb, const float* __restrict__ weight,
+                          TO* __restrict__ out, int width, float eps) {
+  __shared__ float scratch[16];
+  const size_t r = blockIdx.x;
+  float* x = residual + r * width;
+  const TD* ar = a + r * width;
+  const TD* br = b ? b + r * width : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float h = fmaf(sa, to_f32<TD>(ar[i]), x[i]);
+    if (br) h = fmaf(sb, to_f32<TD>(br[i]), h);
+    x[i] = h;
+    ss += h * h;
+  }
+  if (!weight) return;
+  ss = block_sum(ss, scratch);
+  const float scale = 1.0f / sqrtf(ss / (float)width + eps);
+  TO* o = out + r * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x)
+    o[i] = from_f32<TO>(x[i] * scale * weight[i]);   // this thread stored x[i] above
+}
+
+extern "C" int za_scaled_add_rmsnorm(float* residual, const void* a, float sa, const void* b,
+                                     float sb, int delta_dtype, const float* weight, void* out,
+                                     int out_dtype, int n_rows, int width, float eps,
+                                     hipStream_t stream) {
+  if (n_rows == 0) return 0;
+  if (n_rows < 0 || width <= 0 || !residual || !a || (weight && !out)) return ZA_ERR_ARG;
+  dim3 grid(n_rows), block(width <= 256 ? 64 : 256);
+#define ZA_SCALED_ADD(TD, TO)                                                                  \
+  hipLaunchKernelGGL((scaled_add_rmsnorm_kernel<TD, TO>), grid, block, 0, stream, residual,    \
+                     (const TD*)a, sa, (const TD*)b, sb, weight, (TO*)out, width, eps)
+  if (delta_dtype == 0 && out_dtype == 0) ZA_SCALED_ADD(float, float);
+  else if (delta_dtype == 1 && out_dtype == 1) ZA_SCALED_ADD(bf16_t, bf16_t);
+  else if (delta_dtype == 1 && out_dtype == 0) ZA_SCALED_ADD(bf16_t, float);
+  else if (delta_dtype == 0 && out_dtype == 1) ZA_SCALED_ADD(float, bf16_t);
+  else return ZA_ERR_UNSUPPORTED;
+#undef ZA_SCALED_ADD
+  return za_launch_status();
+}

@@ -26,7 +26,11 @@ qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, const int* __restrict__ 
                              const int* __restrict__ slots, const float* __restrict__ q_norm_w,
                              const float* __restrict__ k_norm_w, const float* __restrict__ inv_freq,
                              T* __restrict__ q_out, T* __restrict__ kv_cache, int nh, int nkv, int d,
-                             int rot, int adjacent, float eps, int page_size, int write_kv) {
+                             int rot, int adjacent, float eps, int page_size, int write_kv, int dv,
+                             int row_stride) {
+  // `dv`: width of a value head (queries and keys have `d`); a row of `qkv` holds
+  // nh*d + nkv*d + nkv*dv elements (and may be longer: `row_stride`), a page the keys of
+  // all heads and then the values of all heads.
   __shared__ float vec[4][RK_MAX_D];
   const int t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -38,9 +42,12 @@ qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, const int* __restrict__ 
   float* s = vec[wave];
 
   float ss = 0.f;
+  const bool is_v = active && !is_q && !is_k;
+  const int width = is_v ? dv : d;
   if (active) {
-    const T* src = qkv + ((size_t)t * total + head) * d;
-    for (int i = lane; i < d; i += 64) {
+    const T* src = qkv + (size_t)t * row_stride +
+                   (is_v ? (size_t)(nh + nkv) * d + (size_t)(head - nh - nkv) * dv : (size_t)head * d);
+    for (int i = lane; i < width; i += 64) {
       const float v = to_f32<T>(src[i]);
       s[i] = v;
       ss += v * v;
@@ -78,12 +85,13 @@ qk_norm_rope_kv_write_kernel(const T* __restrict__ qkv, const int* __restrict__ 
     if (slot < 0) return;
     const int page = slot / page_size, off = slot % page_size;
     const int kvh = is_k ? head - nh : head - nh - nkv;
+    T* pg = kv_cache + (size_t)page * nkv * page_size * (d + dv);
     if (is_k) {
-      T* dst = kv_cache + ((((size_t)page * 2) * nkv + kvh) * page_size + off) * d;
+      T* dst = pg + ((size_t)kvh * page_size + off) * d;
       for (int i = lane; i < d; i += 64) dst[i] = from_f32<T>(s[i]);
     } else {
-      T* dst = kv_cache + (((size_t)page * 2 + 1) * nkv + kvh) * page_size * d + off;
-      for (int i = lane; i < d; i += 64) dst[(size_t)i * page_size] = from_f32<T>(s[i]);
+      T* dst = pg + (size_t)nkv * page_size * d + (size_t)kvh * dv * page_size + off;
+      for (int i = lane; i < dv; i += 64) dst[(size_t)i * page_size] = from_f32<T>(s[i]);
     }
   }
 }
@@ -290,12 +298,46 @@ extern "C" int za_qk_norm_rope_kv_write(const void* qkv, const int* positions, c
     hipLaunchKernelGGL((qk_norm_rope_kv_write_kernel<float>), grid, block, 0, stream,
                        (const float*)qkv, positions, slots, q_norm_w, k_norm_w, inv_freq,
                        (float*)q_out, (float*)kv_cache, nh, nkv, d, rot, adjacent, eps, page_size,
-                       write_kv);
+                       write_kv, d, (nh + 2 * nkv) * d);
   } else if (dtype == 1) {
     hipLaunchKernelGGL((qk_norm_rope_kv_write_kernel<bf16_t>), grid, block, 0, stream,
                        (const bf16_t*)qkv, positions, slots, q_norm_w, k_norm_w, inv_freq,
                        (bf16_t*)q_out, (bf16_t*)kv_cache, nh, nkv, d, rot, adjacent, eps,
-                       page_size, write_kv);
+                       page_size, write_kv, d, (nh + 2 * nkv) * d);
+  } else {
+    return ZA_ERR_UNSUPPORTED;
+  }
+  return za_launch_status();
+}
+
+// The same for values of another width than the keys' (`dv`) and rows of `qkv` that hold
+// more than q|k|v (`row_stride` elements a row: a gate's columns behind them, say).
+extern "C" int za_qk_norm_rope_kv_write_wide(const void* qkv, const int* positions,
+                                             const int* slots, const float* q_norm_w,
+                                             const float* k_norm_w, const float* inv_freq,
+                                             void* q_out, void* kv_cache, int dtype, int n_tokens,
+                                             int nh, int nkv, int d, int dv, int row_stride,
+                                             int rot, int adjacent, float eps, int page_size,
+                                             int write_kv, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  if (n_tokens < 0 || nh <= 0 || nkv <= 0 || d <= 0 || dv <= 0 || !qkv || !positions || !q_out ||
+      row_stride < (nh + nkv) * d + nkv * dv)
+    return ZA_ERR_ARG;
+  if (d > RK_MAX_D || dv > RK_MAX_D || rot < 0 || rot > d || (rot % 2) != 0)
+    return ZA_ERR_UNSUPPORTED;
+  if (rot > 0 && !inv_freq) return ZA_ERR_ARG;
+  if (write_kv && (!kv_cache || !slots || page_size <= 0)) return ZA_ERR_ARG;
+  dim3 grid(n_tokens, (nh + 2 * nkv + 3) / 4), block(256);
+  if (dtype == 0) {
+    hipLaunchKernelGGL((qk_norm_rope_kv_write_kernel<float>), grid, block, 0, stream,
+                       (const float*)qkv, positions, slots, q_norm_w, k_norm_w, inv_freq,
+                       (float*)q_out, (float*)kv_cache, nh, nkv, d, rot, adjacent, eps, page_size,
+                       write_kv, dv, row_stride);
+  } else if (dtype == 1) {
+    hipLaunchKernelGGL((qk_norm_rope_kv_write_kernel<bf16_t>), grid, block, 0, stream,
+                       (const bf16_t*)qkv, positions, slots, q_norm_w, k_norm_w, inv_freq,
+                       (bf16_t*)q_out, (bf16_t*)kv_cache, nh, nkv, d, rot, adjacent, eps,
+                       page_size, write_kv, dv, row_stride);
   } else {
     return ZA_ERR_UNSUPPORTED;
   }

@@ -98,7 +98,7 @@ class DecoderModel:
                      for name, family in slots.items()}
             for p in built.values():
                 note(p)
-            self.blocks.append(arrangement(built))
+            self.blocks.append(arrangement(built, **dict(getattr(layer, "params", None) or {})))
             self.mixer_slots.append([n for n, family in slots.items() if family == "mixer"])
         self.final_norm = make("norm", spec.final_norm, ("final_norm",))
         self.head = make("head", spec.lm_head, ("lm_head",))
@@ -155,6 +155,11 @@ class DecoderModel:
         ``library_tuning``: see ``Runtime.library_tuning``."""
         device = device or require_gpu()
         config = load_config(model_dir)
+        if hasattr(config, "with_shapes"):
+            # sizes that config.json leaves to the stored tensors' shapes
+            from ..weights.safetensors_io import Checkpoint
+            ckpt = Checkpoint(model_dir)
+            config = config.with_shapes(lambda name: tuple(ckpt.shape(name)) if name in ckpt else None)
         spec = config.to_spec()
         rt = parts.Runtime(device=device, dtype=run_dtype(dtype), stream_additions=not reproducible,
                            library_tuning=library_tuning)

@@ -86,6 +86,32 @@ _SIGNATURES = {
     ("calibrate", "za_mfma_loop"): [c_int, c_int, c_void_p, c_void_p],
     ("blaslt", "za_lt_matmul"): [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                  c_int, c_void_p, c_size_t, c_void_p],
+    ("rope_kv", "za_qk_norm_rope_kv_write_wide"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                   c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                                   c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                                   c_float, c_int, c_int, c_void_p],
+    ("attention", "za_paged_attention_gated"): [c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                                c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                                c_int, c_void_p, c_void_p, c_int, c_int, c_int,
+                                                c_int, c_int, c_int, c_float, c_int, c_int, c_int,
+                                                c_void_p, c_int, c_int, c_float, c_void_p],
+    ("attention", "za_head_gate"): [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                    c_float, c_void_p],
+    ("activation", "za_clamped_glu"): [c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float,
+                                       c_float, c_void_p],
+    ("norm", "za_scaled_add_rmsnorm"): [c_void_p, c_void_p, c_float, c_void_p, c_float, c_int,
+                                        c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p],
+    ("recurrent", "za_causal_conv_silu"): [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p,
+                                           c_void_p, c_longlong, c_void_p, c_void_p, c_void_p,
+                                           c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    ("recurrent", "za_matrix_recurrence"): [c_int, c_int, c_void_p, c_int, c_int, c_int, c_int,
+                                            c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p,
+                                            c_void_p, c_void_p, c_longlong, c_void_p, c_void_p,
+                                            c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                            c_int, c_int, c_void_p],
+    ("recurrent", "za_gated_group_norm"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int,
+                                           c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
+                                           c_int, c_int, c_float, c_void_p],
 }
 _functions = {}
 
@@ -1334,3 +1360,316 @@ def measured_mfma_rate(repeats: int = 3) -> float:
         if i:
             best = max(best, flops / (start.elapsed_time(stop) * 1e-3))
     return best
+
+
+# ------------------------------------------------- weighted residual additions
+def scaled_add_rmsnorm(residual: torch.Tensor, a: torch.Tensor, scale_a: float,
+                       b: Optional[torch.Tensor] = None, scale_b: float = 0.0,
+                       weight: Optional[torch.Tensor] = None, eps: float = 0.0,
+                       out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """``residual += scale_a * a (+ scale_b * b)`` in 32-bit, in place; with ``weight`` the
+    RMS norm of the sum comes back (``out_dtype``), otherwise ``None``."""
+    n, width = residual.shape
+    _need(residual, "residual", torch.float32, (n, width))
+    _need(a, "a", (torch.float32, torch.bfloat16), (n, width))
+    if b is not None:
+        _need(b, "b", a.dtype, (n, width))
+    out = None
+    if weight is not None:
+        _need(weight, "weight", torch.float32, (width,))
+        out = torch.empty((n, width), dtype=out_dtype or a.dtype, device=residual.device)
+    rc = _fn("norm", "za_scaled_add_rmsnorm")(
+        _ptr(residual), _ptr(a), float(scale_a), _ptr(b), float(scale_b), _code(a.dtype),
+        _ptr(weight), _ptr(out), _code(out.dtype) if out is not None else 0, n, width, float(eps),
+        _stream())
+    _check(rc, "scaled_add_rmsnorm")
+    return out
+
+
+def clamped_glu(gate_up: torch.Tensor, limit: float, alpha: float, up_offset: float) -> torch.Tensor:
+    """``g * sigmoid(alpha * g) * (u + up_offset)`` with ``g = min(gate, limit)`` and
+    ``u = clamp(up, -limit, limit)`` on ``gate_up [T, 2I]``; ``limit <= 0``: unbounded."""
+    _need(gate_up, "gate_up", (torch.float32, torch.bfloat16))
+    if gate_up.dim() != 2 or gate_up.shape[1] % 2:
+        raise KernelError(f"clamped_glu takes [T, 2I], got {tuple(gate_up.shape)}")
+    T, two_i = gate_up.shape
+    out = torch.empty((T, two_i // 2), dtype=gate_up.dtype, device=gate_up.device)
+    rc = _fn("activation", "za_clamped_glu")(_ptr(gate_up), _ptr(out), _code(gate_up.dtype), T,
+                                             two_i // 2, float(limit), float(alpha),
+                                             float(up_offset), _stream())
+    _check(rc, "clamped_glu")
+    return out
+
+
+# ------------------------------------- attention with values of their own width
+def qk_norm_rope_kv_write_wide(qkv: torch.Tensor, positions: torch.Tensor,
+                               slots: Optional[torch.Tensor], q_norm_w: Optional[torch.Tensor],
+                               k_norm_w: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor],
+                               key_plane: Optional[torch.Tensor], value_plane: Optional[torch.Tensor],
+                               num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
+                               rotary_dim: int, adjacent_pairs: bool, eps: float,
+                               write_kv: bool = True) -> torch.Tensor:
+    """As ``qk_norm_rope_kv_write`` for rows ``qkv [T, >= nh*d + nkv*d + nkv*dv]`` (further
+    columns are left alone) and a cache whose pages hold a plane of keys
+    ``[pages, kv_heads, page_size, head_dim]`` followed by a plane of values
+    ``[pages, kv_heads, page_size, value_dim]`` (stored turned round, ``[value_dim][offset]``).
+    Returns the queries ``[T, num_heads, head_dim]``."""
+    T, stride = qkv.shape
+    need = (num_heads + num_kv_heads) * head_dim + num_kv_heads * value_dim
+    _need(qkv, "qkv", (torch.float32, torch.bfloat16))
+    if stride < need:
+        raise KernelError(f"qkv rows hold {stride} elements, fewer than {need}")
+    _need(positions, "positions", torch.int32, (T,))
+    if head_dim > 256 or value_dim > 256:
+        raise KernelError("head widths beyond 256 exceed the kernel's limit")
+    if rotary_dim % 2 or not 0 <= rotary_dim <= head_dim:
+        raise KernelError(f"rotary_dim {rotary_dim} must be even and at most head_dim {head_dim}")
+    for name, w in (("q_norm_w", q_norm_w), ("k_norm_w", k_norm_w)):
+        if w is not None:
+            _need(w, name, torch.float32, (head_dim,))
+    if rotary_dim:
+        _need(inv_freq, "inv_freq", torch.float32, (rotary_dim // 2,))
+    page_size = 0
+    if write_kv:
+        if key_plane is None or value_plane is None or slots is None:
+            raise KernelError("write_kv needs the cache planes and slots")
+        _need(slots, "slots", torch.int32, (T,))
+        page_size = _check_planes(key_plane, value_plane, qkv.dtype, num_kv_heads, head_dim,
+                                  value_dim)
+    q_out = torch.empty((T, num_heads, head_dim), dtype=qkv.dtype, device=qkv.device)
+    rc = _fn("rope_kv", "za_qk_norm_rope_kv_write_wide")(
+        _ptr(qkv), _ptr(positions), _ptr(slots) if write_kv else None, _ptr(q_norm_w),
+        _ptr(k_norm_w), _ptr(inv_freq) if rotary_dim else None, _ptr(q_out),
+        _ptr(key_plane) if write_kv else None, _code(qkv.dtype), T, num_heads, num_kv_heads,
+        head_dim, value_dim, stride, rotary_dim, 1 if adjacent_pairs else 0, float(eps),
+        page_size, 1 if write_kv else 0, _stream())
+    _check(rc, "qk_norm_rope_kv_write_wide")
+    return q_out
+
+
+def _check_planes(key_plane: torch.Tensor, value_plane: torch.Tensor, dtype, nkv: int, d: int,
+                  dv: int) -> int:
+    """The two planes of one cache layer as the kernels index them: a page is the keys of
+    all heads and, right behind them, the values of all heads.  Returns the page size."""
+    for name, t, w in (("key_plane", key_plane, d), ("value_plane", value_plane, dv)):
+        if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != dtype:
+            raise KernelError(f"{name} must be a GPU tensor of {dtype}")
+        if t.dim() != 4 or t.shape[1] != nkv or t.shape[3] != w:
+            raise KernelError(f"{name} has shape {tuple(t.shape)}, expected "
+                              f"[pages, {nkv}, page_size, {w}]")
+    page_size = key_plane.shape[2]
+    per_page = nkv * page_size * (d + dv)
+    if value_plane.shape[2] != page_size or key_plane.stride(0) != per_page \
+            or value_plane.stride(0) != per_page \
+            or key_plane.stride()[1:] != (page_size * d, d, 1) \
+            or value_plane.stride()[1:] != (page_size * dv, dv, 1) \
+            or value_plane.data_ptr() - key_plane.data_ptr() \
+            != nkv * page_size * d * key_plane.element_size():
+        raise KernelError("the key and value planes do not lie as one page after the other")
+    return page_size
+
+
+def paged_attention_gated(q: torch.Tensor, key_plane: torch.Tensor, value_plane: torch.Tensor,
+                          block_table: torch.Tensor, positions: torch.Tensor,
+                          item_seq: torch.Tensor, item_row0: torch.Tensor, item_count: torch.Tensor,
+                          n_items: int, scale: float, window: int = 0, keys_per_split: int = 0,
+                          nsplit: int = 1, gate: Optional[torch.Tensor] = None, gate_col: int = 0,
+                          out_scale: float = 1.0) -> torch.Tensor:
+    """``paged_attention`` for values of their own width: ``q [T, heads, head_dim]``, the
+    cache as a plane of keys and a plane of values (see ``qk_norm_rope_kv_write_wide``);
+    returns ``[T, heads, value_dim]``.  With ``gate [T, columns]`` head ``h`` of token ``t``
+    is multiplied by ``sigmoid(gate[t, gate_col + h]) * out_scale``."""
+    if q.dim() != 3:
+        raise KernelError(f"q must be [T, heads, head_dim], got {tuple(q.shape)}")
+    T, nh, d = q.shape
+    _need(q, "q", (torch.float32, torch.bfloat16))
+    nkv, dv = key_plane.shape[1], value_plane.shape[3]
+    page_size = _check_planes(key_plane, value_plane, q.dtype, nkv, d, dv)
+    if nh % nkv or nh // nkv > ATTENTION_MAX_ROWS:
+        raise KernelError(f"{nh} heads over {nkv} key/value heads: not a whole group of at most "
+                          f"{ATTENTION_MAX_ROWS}")
+    if d % 8 or dv % 8 or d > 256 or dv > 256:
+        raise KernelError(f"head widths {d} and {dv} must be multiples of 8, at most 256")
+    _need(block_table, "block_table", torch.int32)
+    if block_table.dim() != 2:
+        raise KernelError("block_table must be [requests, max_pages]")
+    _need(positions, "positions", torch.int32, (T,))
+    for name, t in (("item_seq", item_seq), ("item_row0", item_row0), ("item_count", item_count)):
+        _need(t, name, torch.int32)
+        if t.numel() < n_items:
+            raise KernelError(f"{name} holds {t.numel()} entries, fewer than {n_items} items")
+    gate_stride = 0
+    if gate is not None:
+        _need(gate, "gate", q.dtype)
+        if gate.dim() != 2 or gate.shape[0] != T or gate_col < 0 or gate_col + nh > gate.shape[1]:
+            raise KernelError(f"gate has shape {tuple(gate.shape)}; columns {gate_col}.."
+                              f"{gate_col + nh} of {T} rows are needed")
+        gate_stride = gate.shape[1]
+    out = torch.empty((T, nh, dv), dtype=q.dtype, device=q.device)
+    part_acc = part_ml = None
+    if nsplit > 1:
+        if keys_per_split <= 0 or keys_per_split % 64:
+            raise KernelError("keys_per_split must be a positive multiple of 64")
+        part_acc = torch.empty((T, nh, nsplit, dv), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((T, nh, nsplit, 2), dtype=torch.float32, device=q.device)
+    rc = _fn("attention", "za_paged_attention_gated")(
+        _ptr(q), _ptr(out), _ptr(key_plane), _ptr(block_table), block_table.shape[1],
+        _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
+        _ptr(part_acc), _ptr(part_ml), _code(q.dtype), nh, nkv, d, dv, page_size, float(scale),
+        int(window), int(keys_per_split), int(nsplit), _ptr(gate), gate_stride, int(gate_col),
+        float(out_scale), _stream())
+    _check(rc, "paged_attention_gated")
+    _note("attention", kernel="plain", rows=T, dtype=q.dtype, nsplit=int(nsplit))
+    return out
+
+
+def head_gate_(out: torch.Tensor, gate: torch.Tensor, gate_col: int, out_scale: float = 1.0) -> torch.Tensor:
+    """``out [T, heads, width]`` times ``sigmoid(gate[t, gate_col + h]) * out_scale``, in place."""
+    T, nh, dv = out.shape
+    _need(out, "out", (torch.float32, torch.bfloat16))
+    _need(gate, "gate", out.dtype)
+    if gate.dim() != 2 or gate.shape[0] != T or gate_col < 0 or gate_col + nh > gate.shape[1]:
+        raise KernelError(f"gate has shape {tuple(gate.shape)}; columns {gate_col}.."
+                          f"{gate_col + nh} of {T} rows are needed")
+    rc = _fn("attention", "za_head_gate")(_ptr(out), _ptr(gate), _code(out.dtype), gate.shape[1],
+                                          int(gate_col), T, nh, dv, float(out_scale), _stream())
+    _check(rc, "head_gate")
+    return out
+
+
+# ------------------------------------------------------- mixers with a matrix state
+CONV_MAX_TAPS = 8
+
+
+def _state_window(state: torch.Tensor, offset: int, count: int, name: str) -> Tuple[int, int]:
+    """``state [slots, floats]`` (32-bit, rows possibly spaced wider than their length):
+    the address of element ``offset`` of slot 0 and the distance between slots."""
+    if not isinstance(state, torch.Tensor) or not state.is_cuda or state.dtype != torch.float32 \
+            or state.dim() != 2 or state.stride(1) != 1:
+        raise KernelError(f"{name} must be a 32-bit GPU tensor [slots, floats]")
+    if offset < 0 or offset + count > state.shape[1]:
+        raise KernelError(f"{name}: floats {offset}..{offset + count} of {state.shape[1]}")
+    return state.data_ptr() + 4 * offset, state.stride(0)
+
+
+def causal_conv_silu(x: torch.Tensor, col0: int, taps: torch.Tensor, bias: Optional[torch.Tensor],
+                     state: torch.Tensor, state_offset: int, token_seq: torch.Tensor,
+                     seq_start: torch.Tensor, slot_id: torch.Tensor) -> torch.Tensor:
+    """``silu(bias + depth-wise causal convolution)`` of columns ``col0 .. col0 + C`` of
+    ``x [T, columns]`` with ``taps [C, L]`` (the last tap meets the current token); the
+    ``L - 1`` inputs before a portion come from ``state[slot, state_offset + c*(L-1) + j]``,
+    which then takes the portion's last inputs.  Returns 32-bit ``[T, C]``."""
+    T, stride = x.shape
+    _need(x, "x", (torch.float32, torch.bfloat16))
+    C, L = taps.shape
+    _need(taps, "taps", torch.float32, (C, L))
+    if not 1 <= L <= CONV_MAX_TAPS:
+        raise KernelError(f"{L} taps: the convolution kernel takes 1 to {CONV_MAX_TAPS}")
+    if col0 < 0 or col0 + C > stride:
+        raise KernelError(f"columns {col0}..{col0 + C} of {stride}")
+    if bias is not None:
+        _need(bias, "bias", torch.float32, (C,))
+    S = slot_id.numel()
+    _need(token_seq, "token_seq", torch.int32, (T,))
+    _need(seq_start, "seq_start", torch.int32, (S + 1,))
+    _need(slot_id, "slot_id", torch.int32, (S,))
+    base, slot_stride = _state_window(state, state_offset, C * (L - 1), "state")
+    out = torch.empty((T, C), dtype=torch.float32, device=x.device)
+    rc = _fn("recurrent", "za_causal_conv_silu")(
+        _ptr(x), _code(x.dtype), stride, int(col0), _ptr(taps), _ptr(bias), base, slot_stride,
+        _ptr(token_seq), _ptr(seq_start), _ptr(slot_id), _ptr(out), T, S, C, L, _stream())
+    _check(rc, "causal_conv_silu")
+    return out
+
+
+def recurrence_plan(dk: int, dv: int) -> Tuple[int, int, int]:
+    """(lanes that split a column's rows, rows per lane, columns per workgroup) for a
+    state of ``dk`` rows and ``dv`` columns."""
+    lanes = 1
+    while lanes * 16 < dk:
+        lanes *= 2
+    if lanes > 64:
+        raise KernelError(f"a state of {dk} rows exceeds the recurrence kernel's limit of 1024")
+    rows = 8 if lanes * 8 >= dk else 16
+    cols = max(1, min(dv, 256 // lanes))
+    return lanes, rows, cols
+
+
+def matrix_recurrence(form: str, conv: torch.Tensor, q_col: int, k_col: int, x_col: int,
+                      proj: torch.Tensor, gate_col: int, decay: Optional[torch.Tensor],
+                      dt_bias: torch.Tensor, A_log: torch.Tensor, D: Optional[torch.Tensor],
+                      state: torch.Tensor, state_offset: int, seq_start: torch.Tensor,
+                      slot_id: torch.Tensor, heads: int, groups: int, dk: int, dv: int) -> torch.Tensor:
+    """The token-by-token walk of csrc/recurrent.hip.  ``form``: ``"ssd"`` or ``"delta"``.
+    ``conv [T, columns]`` 32-bit holds, per token, the vectors read against the state's rows
+    at ``q_col`` and ``k_col`` (``groups`` of ``dk``) and the one written along its columns at
+    ``x_col`` (``heads`` of ``dv``); ``proj [T, columns]`` holds one raw number per head at
+    ``gate_col`` (ssd: the step size, delta: the write strength); ``decay [T, >= heads*dk]``
+    (delta) the raw decays in its first ``heads*dk`` columns.  The state of slot ``s`` lies at ``state[s, state_offset:]`` as
+    ``[heads][dv][dk]``.  Returns 32-bit ``[T, heads*dv]``."""
+    if form not in ("ssd", "delta"):
+        raise KernelError(f"form must be ssd or delta, got {form!r}")
+    delta = form == "delta"
+    T, conv_width = conv.shape
+    _need(conv, "conv", torch.float32)
+    _need(proj, "proj", (torch.float32, torch.bfloat16))
+    if proj.dim() != 2 or proj.shape[0] != T:
+        raise KernelError(f"proj has shape {tuple(proj.shape)}, expected [{T}, columns]")
+    if heads % groups:
+        raise KernelError(f"{heads} heads do not divide into {groups} groups")
+    for name, col, n in (("q_col", q_col, groups * dk), ("k_col", k_col, groups * dk),
+                         ("x_col", x_col, heads * dv)):
+        if col < 0 or col + n > conv_width:
+            raise KernelError(f"{name}: columns {col}..{col + n} of {conv_width}")
+    if gate_col < 0 or gate_col + heads > proj.shape[1]:
+        raise KernelError(f"gate_col: columns {gate_col}..{gate_col + heads} of {proj.shape[1]}")
+    _need(A_log, "A_log", torch.float32, (heads,))
+    if delta:
+        _need(decay, "decay", proj.dtype)
+        if decay.dim() != 2 or decay.shape[0] != T or decay.shape[1] < heads * dk:
+            raise KernelError(f"decay has shape {tuple(decay.shape)}, expected [{T}, >= {heads * dk}]")
+        _need(dt_bias, "dt_bias", torch.float32, (heads * dk,))
+    else:
+        _need(dt_bias, "dt_bias", torch.float32, (heads,))
+        _need(D, "D", torch.float32, (heads,))
+    S = slot_id.numel()
+    _need(seq_start, "seq_start", torch.int32, (S + 1,))
+    _need(slot_id, "slot_id", torch.int32, (S,))
+    base, slot_stride = _state_window(state, state_offset, heads * dk * dv, "state")
+    lanes, rows, cols = recurrence_plan(dk, dv)
+    out = torch.empty((T, heads * dv), dtype=torch.float32, device=conv.device)
+    rc = _fn("recurrent", "za_matrix_recurrence")(
+        1 if delta else 0, _code(proj.dtype), _ptr(conv), conv_width, int(q_col), int(k_col),
+        int(x_col), _ptr(proj), proj.shape[1], int(gate_col), _ptr(decay) if delta else None,
+        decay.shape[1] if delta else 0, _ptr(dt_bias), _ptr(A_log), None if delta else _ptr(D), base, slot_stride,
+        _ptr(seq_start), _ptr(slot_id), _ptr(out), S, heads, groups, dk, dv, lanes, rows, cols,
+        _stream())
+    _check(rc, "matrix_recurrence", f"form={form} heads={heads} dk={dk} dv={dv}")
+    return out
+
+
+def gated_group_norm(y: torch.Tensor, gate: torch.Tensor, gate_col: int, weight: torch.Tensor,
+                     group: int, eps: float, activation: str, gate_first: bool,
+                     out_scale: float = 1.0) -> torch.Tensor:
+    """``y [T, width]`` (32-bit) gated by ``act(gate[t, gate_col + c])`` and RMS-normed over
+    groups of ``group`` columns, times ``weight`` (``[width]``, or shorter and repeated);
+    the gate before the norm (``gate_first``) or after it.  ``activation``: ``silu`` or
+    ``sigmoid``.  Returns ``gate``'s type."""
+    T, width = y.shape
+    _need(y, "y", torch.float32)
+    _need(gate, "gate", (torch.float32, torch.bfloat16))
+    if gate.dim() != 2 or gate.shape[0] != T or gate_col < 0 or gate_col + width > gate.shape[1]:
+        raise KernelError(f"gate has shape {tuple(gate.shape)}; columns {gate_col}.."
+                          f"{gate_col + width} of {T} rows are needed")
+    _need(weight, "weight", torch.float32)
+    if weight.dim() != 1 or width % weight.numel() or group <= 0 or width % group:
+        raise KernelError(f"width {width} against weight {tuple(weight.shape)} and group {group}")
+    if activation not in ("silu", "sigmoid"):
+        raise KernelError(f"activation must be silu or sigmoid, got {activation!r}")
+    out = torch.empty((T, width), dtype=gate.dtype, device=y.device)
+    rc = _fn("recurrent", "za_gated_group_norm")(
+        _ptr(y), _ptr(gate), _code(gate.dtype), gate.shape[1], int(gate_col), _ptr(weight),
+        weight.numel(), _ptr(out), width, 0, T, width, int(group), float(eps),
+        1 if activation == "silu" else 0, 1 if gate_first else 0, float(out_scale), _stream())
+    _check(rc, "gated_group_norm")
+    return out

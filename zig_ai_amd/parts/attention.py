@@ -10,8 +10,14 @@ Per token (/root/reference/src/transformer/hybrid_attn.zig:286-640):
 
 All sizes come from ``params``: ``hidden_size, num_heads, num_kv_heads,
 head_dim, qk_norm, norm_eps, window`` (0 = all keys), ``softmax_scale`` (None =
-1/sqrt(head_dim)), ``bias`` and ``position`` (a nested position-encoding spec or
-None).
+1/sqrt(head_dim)), ``bias`` (true: on all four projections; ``"qkv"``: on the three
+opening ones only) and ``position`` (a nested position-encoding spec or None).
+
+Two more, for designs that need them: ``value_dim`` (values, and with them the
+attention's output per head, of another width than queries and keys) and ``gate``
+(``"head"``: every head's output is multiplied by ``sigmoid(x Wg^T)_h`` before the output
+projection; the gate's rows ride along in the opening projection).  With either, the
+cache is a plane of keys and a plane of values per page.
 """
 
 from __future__ import annotations
@@ -23,7 +29,7 @@ import torch
 
 from ..kernels import ops
 from .base import (Mixer, PagedNeed, Runtime, TensorRule, lookup, register_mixer)
-from .feed_forward import fuse_rows
+from .feed_forward import fuse_rows, pad_rows
 
 # Cutting long contexts pays only when the launch would otherwise leave most of the
 # machine idle (decoding few requests, or a portion of a prompt far into a long
@@ -70,24 +76,31 @@ class GroupedQueryAttention(Mixer):
     def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:
         H, nh, nkv, d = (int(params[k]) for k in
                          ("hidden_size", "num_heads", "num_kv_heads", "head_dim"))
+        dv = int(params.get("value_dim") or d)
         rules = {"q_proj.weight": TensorRule(((nh * d, H),)),
                  "k_proj.weight": TensorRule(((nkv * d, H),)),
-                 "v_proj.weight": TensorRule(((nkv * d, H),)),
-                 "out_proj.weight": TensorRule(((H, nh * d),))}
+                 "v_proj.weight": TensorRule(((nkv * dv, H),)),
+                 "out_proj.weight": TensorRule(((H, nh * dv),))}
+        if params.get("gate") == "head":
+            rules["gate_proj.weight"] = TensorRule(((nh, H),))
         if params.get("qk_norm"):
             rules["q_norm.weight"] = TensorRule(((d,),), role="norm")
             rules["k_norm.weight"] = TensorRule(((d,),), role="norm")
         if params.get("bias"):
             rules["q_proj.bias"] = TensorRule(((nh * d,),), role="bias")
             rules["k_proj.bias"] = TensorRule(((nkv * d,),), role="bias")
-            rules["v_proj.bias"] = TensorRule(((nkv * d,),), role="bias")
-            rules["out_proj.bias"] = TensorRule(((H,),), role="bias")
+            rules["v_proj.bias"] = TensorRule(((nkv * dv,),), role="bias")
+            if params["bias"] != "qkv":
+                rules["out_proj.bias"] = TensorRule(((H,),), role="bias")
         return rules
 
     @classmethod
     def cache_need(cls, params: Mapping[str, Any]):
-        return PagedNeed.kv(int(params["num_kv_heads"]), int(params["head_dim"]),
-                            int(params.get("window") or 0))
+        nkv, d = int(params["num_kv_heads"]), int(params["head_dim"])
+        dv = int(params.get("value_dim") or d)
+        if dv == d:
+            return PagedNeed.kv(nkv, d, int(params.get("window") or 0))
+        return PagedNeed(((nkv, d), (nkv, dv)), int(params.get("window") or 0))
 
     def __init__(self, params, tensors, runtime: Runtime):
         super().__init__(params, tensors, runtime)
@@ -97,6 +110,14 @@ class GroupedQueryAttention(Mixer):
         if self.num_heads % self.num_kv_heads:
             raise ValueError(f"{self.num_heads} heads do not divide into {self.num_kv_heads} groups")
         self.group = self.num_heads // self.num_kv_heads
+        self.value_dim = int(params.get("value_dim") or self.head_dim)
+        if params.get("gate") not in (None, "head"):
+            raise ValueError(f"attention gate must be None or 'head', got {params.get('gate')!r}")
+        self.gated = params.get("gate") == "head"
+        # values of their own width, or a gate: the kernels that take the cache as two planes
+        self.wide = self.gated or self.value_dim != self.head_dim
+        if self.value_dim % 8 or self.value_dim > 256:
+            raise ValueError(f"value_dim {self.value_dim} must be a multiple of 8, at most 256")
         if self.group > ops.ATTENTION_MAX_ROWS:
             raise ValueError(f"{self.group} query heads per key/value head exceed the attention "
                              f"kernel's limit of {ops.ATTENTION_MAX_ROWS}")
@@ -116,14 +137,20 @@ class GroupedQueryAttention(Mixer):
         self.item_granularities = [self.rows_per_item] + (
             [self.mfma_rows_per_item, self.mfma_decode_rows_per_item] if self.mfma else [])
         self.eps = float(params.get("norm_eps", 0.0))
-        self.w_qkv = fuse_rows(tensors["q_proj.weight"], tensors["k_proj.weight"],
-                               tensors["v_proj.weight"])
+        opening = [tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]]
+        self.gate_col = (self.num_heads + self.num_kv_heads) * self.head_dim \
+            + self.num_kv_heads * self.value_dim
+        if self.gated:
+            opening.append(tensors["gate_proj.weight"])
+        self.w_qkv = fuse_rows(*opening)
+        if self.wide:
+            self.w_qkv = pad_rows(self.w_qkv)
         self.w_out = tensors["out_proj.weight"]
         self.b_qkv = self.b_out = None
         if params.get("bias"):
-            self.b_qkv = torch.cat([tensors["q_proj.bias"], tensors["k_proj.bias"],
-                                    tensors["v_proj.bias"]]).contiguous()
-            self.b_out = tensors["out_proj.bias"]
+            b = torch.cat([tensors["q_proj.bias"], tensors["k_proj.bias"], tensors["v_proj.bias"]])
+            self.b_qkv = torch.cat([b, b.new_zeros((self.w_qkv.shape[0] - b.numel(),))]).contiguous()
+            self.b_out = tensors.get("out_proj.bias")
         self.q_norm = tensors.get("q_norm.weight") if params.get("qk_norm") else None
         self.k_norm = tensors.get("k_norm.weight") if params.get("qk_norm") else None
         pos = params.get("position")
@@ -135,8 +162,12 @@ class GroupedQueryAttention(Mixer):
         # step's numbers on the host
         self.graph_safe = self.position is None or bool(getattr(self.position, "graph_safe", False))
         # a decode step's norm, rotation and cache write can run inside its attention kernel
+        if self.wide and self.position is not None and not self.fused_rotation:
+            raise ValueError("an attention with value_dim or gate takes a rotary position "
+                             "encoding or none")
+        self.mfma = self.mfma and self.value_dim == self.head_dim
         self.rotation_in_attention = (
-            self.fused_rotation and runtime.dtype == torch.bfloat16
+            not self.wide and self.fused_rotation and runtime.dtype == torch.bfloat16
             and self.position.rotary_dim == self.head_dim and self.position.pairing != "adjacent")
         ops.check_projection_weight(self.w_qkv, "attention w_qkv")
         ops.check_projection_weight(self.w_out, "attention w_out")
@@ -144,6 +175,8 @@ class GroupedQueryAttention(Mixer):
     def forward(self, x, step, cache, stream: Optional[torch.Tensor] = None):
         nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
         T = x.shape[0]
+        if self.wide:
+            return self._forward_wide(x, step, cache, stream)
         qkv = ops.linear(x, self.w_qkv, self.b_qkv, tune=self.runtime.tune)
         slots = step.slot_mapping[cache.group]
         if self.rotation_in_attention and step.n_tokens == step.n_seqs and cache.writes \
@@ -223,6 +256,50 @@ class GroupedQueryAttention(Mixer):
         if getattr(step, "taps", None) is not None:
             self._leave_taps(step, cache, q, o)
         return ops.linear(o.view(T, nh * d), self.w_out, self.b_out, partial_ok=True,
+                          accumulate=stream, tune=self.runtime.tune)
+
+    def _forward_wide(self, x, step, cache, stream: Optional[torch.Tensor] = None):
+        """Values of their own width and/or a gate per head: the opening projection is
+        q | k | v | gate, the cache a plane of keys and a plane of values."""
+        nh, nkv, d, dv = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
+        T = x.shape[0]
+        qkv = ops.linear(x, self.w_qkv, self.b_qkv, tune=self.runtime.tune)
+        key_plane, value_plane = cache.planes
+        rot = self.position.rotary_dim if self.position is not None else 0
+        q = ops.qk_norm_rope_kv_write_wide(
+            qkv, step.positions, step.slot_mapping[cache.group], self.q_norm, self.k_norm,
+            self.position.inv_freq if rot else None, key_plane, value_plane, nh, nkv, d, dv, rot,
+            bool(rot) and self.position.pairing == "adjacent", self.eps, write_kv=cache.writes)
+        table = step.block_tables[cache.group]
+        gate = qkv if self.gated else None
+        # (ranges are cut at absolute key positions: behind a window nearly all of them
+        # would be empty, so a windowed layer's contexts are never cut)
+        def split(n_items, **kw):
+            return (0, 1) if self.window else plan_split(n_items, nkv, step.max_keys, **kw)
+        if self.mfma and cache.kv is not None and cache.kv.shape[3] % 4 == 0:
+            if step.n_tokens > step.n_seqs:
+                items = step.attention_items(self.mfma_rows_per_item)
+                keys, nsplit = split(items[3], target=BUSY_WORKGROUPS)
+                o = ops.paged_attention_mfma(q, cache.kv, table, step.positions, *items,
+                                             self.scale, self.window, keys, nsplit,
+                                             tile_keys=128 if d == 64 else 64)
+            else:
+                keys, nsplit = split(step.n_seqs)
+                o = ops.paged_attention_decode_mfma(q, cache.kv, table, step.positions, None,
+                                                    None, None, step.n_seqs, self.scale,
+                                                    self.window, keys, nsplit)
+            if gate is not None:
+                ops.head_gate_(o, gate, self.gate_col)
+        else:
+            item_seq, item_row0, item_count, n_items = step.attention_items(self.rows_per_item)
+            keys, nsplit = split(n_items)
+            o = ops.paged_attention_gated(q, key_plane, value_plane, table, step.positions,
+                                          item_seq, item_row0, item_count, n_items, self.scale,
+                                          self.window, keys, nsplit, gate, self.gate_col)
+        if getattr(step, "taps", None) is not None:
+            step.taps["q"] = q.clone()
+            step.taps["o"] = o.clone()
+        return ops.linear(o.view(T, nh * dv), self.w_out, self.b_out, partial_ok=True,
                           accumulate=stream, tune=self.runtime.tune)
 
     def _leave_taps(self, step, cache, q: torch.Tensor, o: torch.Tensor) -> None:

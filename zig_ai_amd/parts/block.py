@@ -60,3 +60,71 @@ def apply_normed(norm, part, residual: torch.Tensor, pending: Optional[torch.Ten
 
 
 register_arrangement(PreNormResidualBlock.kind, PreNormResidualBlock)
+
+
+class ScaledResidualBlock:
+    """A pre-norm block whose parts enter the stream with weights, and which may run two
+    mixers side by side on the same normed input and may lack the feed-forward:
+
+        h = x + m * (a * left(norm1(x)) + b * right(norm1(x)));   y = h + m * ff(norm2(h))
+
+    ``m`` (``residual_scale``), ``a`` and ``b`` (``mixer_scales``) are the layer's
+    ``params``.  The weighted sums are taken in 32-bit by one kernel that also runs the
+    norm that follows inside the block; nothing is left pending."""
+
+    mixers = ("mixer",)
+    has_feed_forward = True
+
+    def __init__(self, parts, residual_scale: float = 1.0, mixer_scales=None):
+        self.parts = dict(parts)
+        self.mixer_norm = parts["mixer_norm"]
+        self.mixer_parts = [parts[name] for name in self.mixers]
+        self.feed_forward_norm = parts.get("feed_forward_norm")
+        self.feed_forward = parts.get("feed_forward")
+        self.residual_scale = float(residual_scale)
+        scales = list(mixer_scales) if mixer_scales is not None else [1.0] * len(self.mixers)
+        if len(scales) != len(self.mixers) or not 1 <= len(scales) <= 2:
+            raise ValueError(f"{len(self.mixers)} mixers need as many scales, got {scales!r}")
+        self.mixer_scales = [float(s) * self.residual_scale for s in scales]
+
+    def forward(self, residual: torch.Tensor, pending: Optional[torch.Tensor], step,
+                cache) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+        from ..kernels import ops
+        h = self.mixer_norm.add_forward(residual, pending)
+        if len(self.mixers) == 1:
+            outs = [self.mixer_parts[0].forward(h, step, cache)]
+        else:
+            outs = [part.forward(h, step, cache[name])
+                    for name, part in zip(self.mixers, self.mixer_parts)]
+        second = (outs[1], self.mixer_scales[1]) if len(outs) == 2 else (None, 0.0)
+        if not self.has_feed_forward:
+            ops.scaled_add_rmsnorm(residual, outs[0], self.mixer_scales[0], *second)
+            return residual, None
+        norm = self.feed_forward_norm
+        if hasattr(norm, "weight") and hasattr(norm, "eps"):
+            h = ops.scaled_add_rmsnorm(residual, outs[0], self.mixer_scales[0], *second,
+                                       weight=norm.weight, eps=norm.eps, out_dtype=h.dtype)
+        else:
+            ops.scaled_add_rmsnorm(residual, outs[0], self.mixer_scales[0], *second)
+            h = norm.forward(residual)
+        y = self.feed_forward.forward(h, step)
+        ops.scaled_add_rmsnorm(residual, y, self.residual_scale)
+        return residual, None
+
+
+def _scaled_variant(kind: str, mixers, feed_forward: bool):
+    slots = {"mixer_norm": "norm"}
+    slots.update({name: "mixer" for name in mixers})
+    if feed_forward:
+        slots.update({"feed_forward_norm": "norm", "feed_forward": "feed_forward"})
+    cls = type("ScaledResidualBlock_" + kind, (ScaledResidualBlock,),
+               {"kind": kind, "slots": slots, "mixers": tuple(mixers),
+                "has_feed_forward": feed_forward})
+    register_arrangement(kind, cls)
+    return cls
+
+
+_scaled_variant("scaled_residual", ("mixer",), True)
+_scaled_variant("scaled_residual_no_ff", ("mixer",), False)
+_scaled_variant("scaled_residual_parallel", ("left", "right"), True)
+_scaled_variant("scaled_residual_parallel_no_ff", ("left", "right"), False)

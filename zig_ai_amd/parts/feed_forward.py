@@ -21,6 +21,24 @@ def fuse_rows(*mats: torch.Tensor) -> torch.Tensor:
     return torch.cat(mats, dim=0).contiguous()
 
 
+def pad_rows(w: torch.Tensor, multiple: int = 8) -> torch.Tensor:
+    """``w [N, K]`` with zero rows appended up to a multiple: a fused projection's output
+    rows then start on 16-byte boundaries in either storage type."""
+    extra = -w.shape[0] % multiple
+    if not extra:
+        return w
+    return torch.cat([w, w.new_zeros((extra,) + tuple(w.shape[1:]))], dim=0).contiguous()
+
+
+def pad_columns(w: torch.Tensor, multiple: int = 8) -> torch.Tensor:
+    """``w [N, K]`` with zero columns appended up to a multiple (a product's input width
+    has to be one; the inputs that meet the new columns must be zero as well)."""
+    extra = -w.shape[1] % multiple
+    if not extra:
+        return w
+    return torch.cat([w, w.new_zeros((w.shape[0], extra))], dim=1).contiguous()
+
+
 class SwiGLU(FeedForward):
     kind = "swiglu"
     graph_safe = True
@@ -56,4 +74,40 @@ class SwiGLU(FeedForward):
         return ops.linear(a, self.down, partial_ok=True, accumulate=stream, tune=self.runtime.tune)
 
 
+class ClampedGLU(FeedForward):
+    """A gated unit whose two inputs are bounded before they meet:
+
+        g = min(x Wg^T, limit);  u = clamp(x Wu^T, -limit, limit)
+        y = (g * sigmoid(alpha * g) * (u + up_offset)) Wd^T
+
+    ``limit`` (none if 0), ``alpha`` and ``up_offset`` come from ``params``.  Gate and up
+    weights are one matrix, as in ``SwiGLU``; the activation is a kernel of its own."""
+
+    kind = "clamped_glu"
+    graph_safe = True
+    kernel_sources = ("gemm", "activation")
+
+    @classmethod
+    def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:
+        H, I = int(params["hidden_size"]), int(params["intermediate_size"])
+        return {"gate.weight": TensorRule(((I, H),)), "up.weight": TensorRule(((I, H),)),
+                "down.weight": TensorRule(((H, I),))}
+
+    def __init__(self, params, tensors, runtime: Runtime):
+        super().__init__(params, tensors, runtime)
+        self.limit = float(params.get("limit") or 0.0)
+        self.alpha = float(params.get("alpha", 1.0))
+        self.up_offset = float(params.get("up_offset", 0.0))
+        self.gate_up = fuse_rows(tensors["gate.weight"], tensors["up.weight"])
+        self.down = tensors["down.weight"]
+        ops.check_projection_weight(self.gate_up, "feed_forward gate_up")
+        ops.check_projection_weight(self.down, "feed_forward down")
+
+    def forward(self, x, step=None):
+        a = ops.clamped_glu(ops.linear(x, self.gate_up, tune=self.runtime.tune), self.limit,
+                            self.alpha, self.up_offset)
+        return ops.linear(a, self.down, tune=self.runtime.tune)
+
+
 register_feed_forward(SwiGLU.kind, SwiGLU)
+register_feed_forward(ClampedGLU.kind, ClampedGLU)

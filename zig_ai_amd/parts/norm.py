@@ -1,6 +1,9 @@
 """RMSNorm as a part.  ``out = x / sqrt(mean(x^2) + eps) * weight`` in 32-bit
 (/root/reference/src/transformer/norm.zig:6-33); ``add_forward`` fuses the
-residual add that precedes the norm in a pre-norm block."""
+residual add that precedes the norm in a pre-norm block.  With ``weight_offset`` the
+stored tensor is the weight's distance from that number (a weight kept around zero and
+used as ``1 + w`` has ``weight_offset = 1``); the sum is taken once, in 32-bit, when the
+part is built."""
 
 from __future__ import annotations
 
@@ -19,13 +22,18 @@ class RMSNorm(Norm):
 
     @classmethod
     def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:
-        return {"weight": TensorRule(((int(params["width"]),),), role="norm")}
+        # (a weight stored as an offset starts around zero, like a bias)
+        role = "bias" if float(params.get("weight_offset", 0.0)) else "norm"
+        return {"weight": TensorRule(((int(params["width"]),),), role=role)}
 
     def __init__(self, params, tensors, runtime: Runtime):
         super().__init__(params, tensors, runtime)
         self.width = int(params["width"])
         self.eps = float(params["eps"])
         self.weight = tensors["weight"]
+        offset = float(params.get("weight_offset", 0.0))
+        if offset:
+            self.weight = (self.weight.float() + offset).contiguous()
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         shape = x.shape
