@@ -33,7 +33,7 @@
 #include "common.h"
 
 #define RC_MAX_TAPS 8
-#define RC_CHUNK 16          // tokens prepared into LDS at a time
+#define RC_CHUNK 16          // tokens prepared into LDS at a time, at most
 
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
@@ -159,6 +159,7 @@ struct RecurrenceArgs {
   float* out;             // [T][H*dv] 32-bit
   int H, G, dk, dv, P;
   int cols_per_block;     // columns of S a workgroup keeps (grid.z covers dv)
+  int chunk;              // tokens prepared into LDS at a time (what fits)
 };
 
 // LDS index of key channel i when a lane owns R consecutive channels: one float of
@@ -177,11 +178,12 @@ matrix_recurrence_kernel(RecurrenceArgs a) {
   const bool owner = tid / P < a.cols_per_block && col < dv;
   const int kpad = lds_at<R>(dk - 1) + 1;
   // LDS: per chunk token: kvec[kpad], qvec[kpad], (delta) gvec[kpad], xvec[dv], 2 scalars
+  const int CH = a.chunk;
   float* Kc = lds;
-  float* Qc = Kc + RC_CHUNK * kpad;
-  float* Gc = Qc + RC_CHUNK * kpad;
-  float* Xc = Gc + (DELTA ? RC_CHUNK * kpad : 0);
-  float* Sc = Xc + RC_CHUNK * dv;          // [RC_CHUNK][2]: SSD (decay, dt); delta (beta, -)
+  float* Qc = Kc + CH * kpad;
+  float* Gc = Qc + CH * kpad;
+  float* Xc = Gc + (DELTA ? CH * kpad : 0);
+  float* Sc = Xc + CH * dv;                // [chunk][2]: SSD (decay, dt); delta (beta, -)
 
   const int start = a.seq_start[s], n = a.seq_start[s + 1] - start;
   float* st = a.state + (size_t)a.slot_id[s] * a.slot_stride + ((size_t)h * dv + col) * dk;
@@ -197,8 +199,8 @@ matrix_recurrence_kernel(RecurrenceArgs a) {
   const T* proj = (const T*)a.proj;
   const T* decay = (const T*)a.decay;
 
-  for (int c0 = 0; c0 < n; c0 += RC_CHUNK) {
-    const int cn = n - c0 < RC_CHUNK ? n - c0 : RC_CHUNK;
+  for (int c0 = 0; c0 < n; c0 += CH) {
+    const int cn = n - c0 < CH ? n - c0 : CH;
     __syncthreads();     // the chunk before has been walked
     if (DELTA) {
       // unit vectors: a wave takes (token, q or k) pairs in turn
@@ -296,11 +298,13 @@ matrix_recurrence_kernel(RecurrenceArgs a) {
 }
 
 template <typename T, bool DELTA>
-static int launch_recurrence(const RecurrenceArgs& a, int n_seqs, int R, hipStream_t stream) {
+static int launch_recurrence(RecurrenceArgs a, int n_seqs, int R, hipStream_t stream) {
   const int threads = (a.cols_per_block * a.P + 63) / 64 * 64;
   const int kpad = a.dk + (a.dk - 1) / R + 1;
-  const size_t lds = sizeof(float) * ((size_t)RC_CHUNK * kpad * (DELTA ? 3 : 2) +
-                                      (size_t)RC_CHUNK * a.dv + RC_CHUNK * 2);
+  const size_t per_token = sizeof(float) * ((size_t)kpad * (DELTA ? 3 : 2) + a.dv + 2);
+  a.chunk = RC_CHUNK;
+  while (a.chunk > 1 && a.chunk * per_token > 64 * 1024) a.chunk /= 2;
+  const size_t lds = a.chunk * per_token;
   if (lds > 64 * 1024) return ZA_ERR_UNSUPPORTED;
   dim3 grid(n_seqs, a.H, (a.dv + a.cols_per_block - 1) / a.cols_per_block), block(threads);
 #define ZA_RECURRENCE(RR)                                                                    \
@@ -335,7 +339,7 @@ extern "C" int za_matrix_recurrence(int form, int dtype, const float* conv, int 
     return ZA_ERR_ARG;
   RecurrenceArgs a{conv, conv_width, q_col, k_col, x_col, proj, proj_stride, gate_col, decay,
                    decay_stride, dt_bias, A_log, D, state, slot_stride, seq_start, slot_id, out,
-                   H, G, dk, dv, lanes, cols_per_block};
+                   H, G, dk, dv, lanes, cols_per_block, RC_CHUNK};
   if (dtype == 0)
     return form ? launch_recurrence<float, true>(a, n_seqs, rows_per_lane, stream)
                 : launch_recurrence<float, false>(a, n_seqs, rows_per_lane, stream);

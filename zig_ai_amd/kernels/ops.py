@@ -370,6 +370,15 @@ def check_projection_weight(weight: torch.Tensor, what: str) -> None:
             "32-bit or run with float32")
 
 
+def projection_weight(weight: torch.Tensor) -> torch.Tensor:
+    """``weight`` as the products can take it: a bfloat16 matrix whose input width is no
+    multiple of 8 is widened to 32-bit (the all-32-bit kernel takes any width, with
+    activations of either type)."""
+    if weight.dtype == torch.bfloat16 and weight.shape[1] % 8:
+        return weight.float().contiguous()
+    return weight
+
+
 def _k_splits(M: int, N: int, K: int) -> int:
     """Into how many ranges K is cut when the consumer accepts partial sums:
     enough to give every compute unit work when N alone is too small.  Measured

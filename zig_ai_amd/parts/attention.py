@@ -121,8 +121,10 @@ class GroupedQueryAttention(Mixer):
         if self.group > ops.ATTENTION_MAX_ROWS:
             raise ValueError(f"{self.group} query heads per key/value head exceed the attention "
                              f"kernel's limit of {ops.ATTENTION_MAX_ROWS}")
-        if self.head_dim % 16 or self.head_dim > 256:
-            raise ValueError(f"head_dim {self.head_dim} must be a multiple of 16, at most 256")
+        # (the kernels that take the cache as two planes read eight elements at a time)
+        multiple = 8 if self.wide else 16
+        if self.head_dim % multiple or self.head_dim > 256:
+            raise ValueError(f"head_dim {self.head_dim} must be a multiple of {multiple}, at most 256")
         # tokens per work item of the two attention kernels
         self.rows_per_item = max(1, ops.ATTENTION_MAX_ROWS // self.group)
         self.mfma_rows_per_item = max(1, ops.ATTENTION_MFMA_ROWS // self.group)
@@ -143,9 +145,10 @@ class GroupedQueryAttention(Mixer):
         if self.gated:
             opening.append(tensors["gate_proj.weight"])
         self.w_qkv = fuse_rows(*opening)
-        if self.wide:
-            self.w_qkv = pad_rows(self.w_qkv)
         self.w_out = tensors["out_proj.weight"]
+        if self.wide:
+            self.w_qkv = ops.projection_weight(pad_rows(self.w_qkv))
+            self.w_out = ops.projection_weight(self.w_out)
         self.b_qkv = self.b_out = None
         if params.get("bias"):
             b = torch.cat([tensors["q_proj.bias"], tensors["k_proj.bias"], tensors["v_proj.bias"]])

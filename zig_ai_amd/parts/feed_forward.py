@@ -98,10 +98,8 @@ class ClampedGLU(FeedForward):
         self.limit = float(params.get("limit") or 0.0)
         self.alpha = float(params.get("alpha", 1.0))
         self.up_offset = float(params.get("up_offset", 0.0))
-        self.gate_up = fuse_rows(tensors["gate.weight"], tensors["up.weight"])
-        self.down = tensors["down.weight"]
-        ops.check_projection_weight(self.gate_up, "feed_forward gate_up")
-        ops.check_projection_weight(self.down, "feed_forward down")
+        self.gate_up = ops.projection_weight(fuse_rows(tensors["gate.weight"], tensors["up.weight"]))
+        self.down = ops.projection_weight(tensors["down.weight"])
 
     def forward(self, x, step=None):
         a = ops.clamped_glu(ops.linear(x, self.gate_up, tune=self.runtime.tune), self.limit,

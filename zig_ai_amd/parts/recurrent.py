@@ -80,8 +80,8 @@ class StateSpaceDuality(Mixer):
         self.heads, self.head_dim, self.state_size, self.groups, self.taps = H, P, N, G, L
         self.inner = H * P
         self.eps = float(params["norm_eps"])
-        self.w_in = pad_rows(tensors["in_proj.weight"])
-        self.w_out = tensors["out_proj.weight"]
+        self.w_in = ops.projection_weight(pad_rows(tensors["in_proj.weight"]))
+        self.w_out = ops.projection_weight(tensors["out_proj.weight"])
         self.conv_w = tensors["conv.weight"]
         self.conv_b = tensors["conv.bias"]
         self.dt_bias, self.A_log, self.D = tensors["dt_bias"], tensors["A_log"], tensors["D"]
@@ -165,11 +165,12 @@ class GatedDeltaRule(Mixer):
         top = torch.cat([up_a, up_a.new_zeros((up_a.shape[0], up_g.shape[1]))], dim=1)
         bottom = torch.cat([up_g.new_zeros((up_g.shape[0], up_a.shape[1])), up_g], dim=1)
         self.w_up = pad_rows(torch.cat([top, bottom], dim=0))
+        self.w_in = ops.projection_weight(self.w_in)
         self.conv_w = torch.cat([tensors["q_conv.weight"], tensors["k_conv.weight"],
                                  tensors["v_conv.weight"]], dim=0).contiguous()
         self.A_log, self.dt_bias = tensors["A_log"], tensors["dt_bias"]
         self.norm_w = tensors["norm.weight"]
-        self.w_out = tensors["out_proj.weight"]
+        self.w_out = ops.projection_weight(tensors["out_proj.weight"])
         self.conv_state = (2 * G * d + H * dv) * (L - 1)
         for w, what in ((self.w_in, "in"), (self.w_up, "low-rank up"), (self.w_out, "out")):
             ops.check_projection_weight(w, f"gated_delta {what} projection")
