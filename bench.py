@@ -3,6 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
     python bench.py --shape 2.6b --prompt-len 6144        # another LFM2 shape, same measurement
     python bench.py --shape 350m --workload serve         # 64 requests through the scheduler
+    python bench.py --workload compare                    # Rudilix beside LFM2 at equal sizes
 
 Default run: the layer sizes of the LFM2-1.2B shape (16 layers, hidden 2048, vocabulary 65,536)
 with random bfloat16 weights N(0, 0.02), a batch of 8 requests, each prefilled
@@ -25,6 +26,12 @@ shape (no timing of candidates, which allocates, frees and waits inside the firs
 and weights drawn with one kernel a tensor (other values than the default run's).
 The model is ``DecoderModel.from_random(cfg, seed=0)``: the tensors that
 ``write_random_model(cfg, folder, seed=0)`` stores, drawn on the device.
+
+``--workload compare``: a Rudilix model (sliding-window attention beside the gated delta
+rule, state-space and delta layers) and an LFM2 model of the same width, depth,
+feed-forward width and vocabulary, attention where the other has it, both with random
+weights: a 2,048-token prefill and decode steps of a batch of 8 at that context, per
+width (``--compare-widths``), as one JSON line.
 """
 
 import argparse
@@ -124,6 +131,106 @@ def serve(cfg, name, n_requests, new_tokens, portion_graphs=False, chunk_size=No
         "data": "synthetic token ids; random weights N(0, 0.02)"}
 
 
+def rudilix_shape(width, layers, vocab):
+    """Layer sizes in the manner of a real model of this design: every fourth layer the
+    attention (window 1,024) beside the delta rule, state-space layers with twice the
+    width inside, delta layers between them; feed-forward of four times the width."""
+    heads = width // 128
+    attention = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128,
+                 "scale": 128 ** -0.5, "mask": {"size": 1024}, "rot": {"dims": 64, "base": 1e6}}
+    delta = {"heads": heads, "kv_heads": heads, "dim": 128, "vdim": 128, "conv": 4,
+             "decay_rank": 64, "gate_rank": 64}
+    ssd = {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 1, "norm_groups": 1,
+           "conv": 4}
+    mlp = {"kind": "dense", "ff": 4 * width, "limit": 7.0}
+    kinds = ["parallel", "mamba2", "channel_delta", "mamba2"]
+    out = []
+    for i in range(layers):
+        kind = kinds[i % 4]
+        mixer = {"left": attention, "right": dict(delta, heads=heads // 2, kv_heads=heads // 2),
+                 "left_scale": 1.0, "right_scale": 1.0} if kind == "parallel" \
+            else (ssd if kind == "mamba2" else delta)
+        out.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Rudilix", "vocab": vocab, "width": width, "residual_mult": 1.0,
+            "norm": {"eps": 1e-5}, "layers": out, "max_position_embeddings": 128000}
+
+
+def compare(widths, layers, batch, prompt_len, steps, warmup) -> dict:
+    """Prefill and decode throughput of Rudilix and of LFM2 at equal sizes."""
+    import torch
+    from zig_ai_amd.engine import DecoderModel, ModelRunner, StepEntry
+    from zig_ai_amd.kernels import ops
+    torch.cuda.set_device(0)
+    vocab, page = 65536, 16
+    gen = torch.Generator().manual_seed(4321)
+
+    def tokens(n):
+        return torch.randint(0, vocab, (n,), generator=gen).tolist()
+
+    def measure(cfg):
+        model = DecoderModel.from_random(cfg, seed=0, dtype="bfloat16", quick=True)
+        out = {"weight_bytes": count_bytes(model)}
+        # ---- prefill: whole prompts of prompt_len tokens, one a step
+        runner = ModelRunner(model, page_size=page, num_pages=4 * (prompt_len // page + 1), num_slots=4)
+
+        def one(name):
+            runner.admit(name)
+            runner.step([StepEntry(name, tokens(prompt_len), [prompt_len - 1])])
+            runner.release(name)
+        for r in range(3):
+            one(("w", r))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for r in range(6):
+            one(("p", r))
+        torch.cuda.synchronize()
+        seconds = (time.perf_counter() - t0) / 6
+        out["prefill"] = {"tokens": prompt_len, "ms": seconds * 1e3, "tokens_per_s": prompt_len / seconds}
+        del runner
+        torch.cuda.empty_cache()
+        # ---- decode: a batch at that context, steps issued as generation issues them
+        need = batch * ((prompt_len + steps + warmup + 2 + page - 1) // page + 1)
+        runner = ModelRunner(model, page_size=page, num_pages=need, num_slots=batch)
+        last = []
+        for r in range(batch):
+            runner.admit(r)
+            logits = runner.step([StepEntry(r, tokens(prompt_len), [prompt_len - 1])])
+            last.append(int(ops.argmax(logits)[0]))
+        requests = list(range(batch))
+        greedy = lambda logits, i: ops.argmax(logits)
+
+        def run(cur, device, n):
+            done = 0
+            while done < n:
+                drawn = runner.decode_steps(requests, cur, min(8, n - done), greedy, device_tokens=device)
+                device, cur = drawn[drawn.shape[0] - 1], None
+                done += drawn.shape[0]
+            return device
+        device = run(last, None, warmup)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run(None, device, steps)
+        torch.cuda.synchronize()
+        seconds = (time.perf_counter() - t0) / steps
+        out["decode"] = {"batch": batch, "ctx": prompt_len, "ms_per_step": seconds * 1e3,
+                         "tokens_per_s": batch / seconds,
+                         "weights_GBps": out["weight_bytes"] / seconds / 1e9,
+                         "graphs": runner.graphs is not None}
+        del runner, model
+        torch.cuda.empty_cache()
+        return out
+
+    result = {"workload": "compare", "dtype": "bf16", "data": "synthetic", "layers": layers,
+              "batch": batch, "prompt_len": prompt_len, "steps": steps, "warmup": warmup, "widths": {}}
+    for width in widths:
+        new = rudilix_shape(width, layers, vocab)
+        attention_at = tuple(i for i, l in enumerate(new["layers"]) if l["type"] == "parallel")
+        old = _shape(width, width // 64, max(1, width // 256), 4 * width, layers, attention_at)
+        old.update(block_auto_adjust_ff_dim=False, vocab_size=vocab, tie_embedding=False)
+        result["widths"][str(width)] = {"rudilix": measure(new), "lfm2": measure(old)}
+    return result
+
+
 def count_bytes(model):
     """Bytes of every weight a decode step reads once (a tied head reads the
     embedding table once; the embedding gather itself reads a few rows)."""
@@ -167,7 +274,10 @@ def main() -> int:
                     help="run fewer layers than the configuration has (both numbers are reported)")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="1.2b",
                     help="layer sizes: LFM2-1.2B (the default run), 350M or 2.6B")
-    ap.add_argument("--workload", choices=["steps", "serve"], default="steps",
+    ap.add_argument("--compare-widths", default="1024,2048",
+                    help="--workload compare: the widths, with commas between them")
+    ap.add_argument("--compare-layers", type=int, default=8, help="--workload compare: layers")
+    ap.add_argument("--workload", choices=["steps", "serve", "compare"], default="steps",
                     help="steps: decode steps and one prefill (the default run); serve: 64 "
                          "requests with prompts of 128-2048 tokens and 256 new tokens each "
                          "through the scheduler")
@@ -200,6 +310,11 @@ def main() -> int:
 
     torch.cuda.set_device(0)
     cfg = dict(SHAPES[args.shape])
+    if args.workload == "compare":
+        print(json.dumps(compare([int(w) for w in args.compare_widths.split(",")],
+                                 args.compare_layers, args.batch, args.prompt_len, args.steps,
+                                 args.warmup)), flush=True)
+        return 0
     if args.workload == "serve":
         print(json.dumps(serve(cfg, args.shape.upper(), args.requests, args.new_tokens,
                                args.portion_graphs, args.chunk_size)), flush=True)
