@@ -26,7 +26,7 @@ pytestmark = pytest.mark.gpu
 
 F32_BOUND = 1e-4
 BF16_MEDIAN, BF16_DECILE, BF16_WORST = 0.04, 0.12, 0.6
-BF16_BETWEEN_MEDIAN, BF16_BETWEEN_WORST = 4e-3, 0.1       # one schedule against another
+BF16_BETWEEN_MEDIAN, BF16_BETWEEN_WORST = 1e-3, 0.03      # one schedule against another (measured 0 and 0.006)
 
 
 def build(cfg, seed=0, dtype="float32", tensors=None):

@@ -17,12 +17,13 @@
 //          g = exp(-exp(A_log) * softplus(raw + dt_bias))   (one per head and key channel)
 //          q, k made unit vectors (x / sqrt(sum x^2 + 1e-6)), q times dk^(-1/2),
 //          beta = sigmoid(raw)
-//    A column of S never meets another column: a thread (or P neighbouring lanes that
-//    split the rows) keeps one column in registers across all tokens of the portion,
-//    reads it from the slot at the start and stores it at the end.  The slot holds S
-//    turned round, [head][column][row], so that a lane's rows are consecutive floats.
-//    The per-token vectors of a chunk of tokens are prepared by the whole workgroup
-//    into LDS (norms, decays, gates), then the tokens are walked in order.
+//    A column of S never meets another column: P neighbouring lanes that split its rows
+//    keep one column in registers across all tokens of the portion, read it from the
+//    slot at the start and store it at the end.  The slot holds S turned round,
+//    [head][column][row], so that a lane's rows are consecutive floats.  What a token
+//    brings that does not depend on the state (unit vectors, decays, gates) is computed
+//    beforehand, for all tokens at once; a workgroup is one wave that walks the tokens in
+//    order with the next tokens' vectors already on their way.
 //
 // 3. gated_group_norm: y * act(gate) and an RMS norm over equal groups of columns, the
 //    gate before or after the norm:
@@ -33,7 +34,6 @@
 #include "common.h"
 
 #define RC_MAX_TAPS 8
-#define RC_CHUNK 16          // tokens prepared into LDS at a time, at most
 
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
@@ -136,217 +136,345 @@ extern "C" int za_causal_conv_silu(const void* x, int dtype, int x_stride, int c
 // What the two forms read, per token row t:
 //   conv   [T][conv_width] 32-bit: the convolution's output.
 //          SSD:   x of head h at x_col + h*dv, b of group g at k_col + g*dk, c at q_col + g*dk
-//          delta: q of key head g at q_col + g*dk, k at k_col + g*dk, v of head h at x_col + h*dv
-//   proj   [T][proj_stride] storage type: the opening projection's raw output.
-//          SSD:   dt of head h at gate_col + h
-//          delta: beta of head h at gate_col + h
-//   decay  [T][decay_stride] storage type (delta only): the decay's raw value per head and key
-//          channel, head h's at columns h*dk
+//          delta: v of head h at x_col + h*dv (q and k come prepared, see below)
+//   proj   [T][proj_stride] storage type (SSD): the raw step size of head h at gate_col + h
+//   prep   [T][prep_width] 32-bit (delta), written by delta_prepare_kernel:
+//          unit q of key head g at g*dk (times dk^-1/2), unit k at G*dk + g*dk, the decay of
+//          head h and key channel i at 2*G*dk + h*dk + i, beta of head h at 2*G*dk + H*dk + h
 struct RecurrenceArgs {
   const float* conv;
   int conv_width, q_col, k_col, x_col;
   const void* proj;
-  int proj_stride, gate_col;
-  const void* decay;
-  int decay_stride;
-  const float* dt_bias;   // SSD: [H]; delta: [H*dk]
-  const float* A_log;     // [H]
+  int proj_stride, gate_col, proj_bf16;
+  const float* prep;
+  int prep_width;
+  const float* dt_bias;   // SSD: [H]
+  const float* A_log;     // SSD: [H]
   const float* D;         // SSD: [H]
   float* state;           // per slot [H][dv][dk]
   long long slot_stride;
   const int* seq_start;
   const int* slot_id;
   float* out;             // [T][H*dv] 32-bit
-  int H, G, dk, dv, P;
-  int cols_per_block;     // columns of S a workgroup keeps (grid.z covers dv)
-  int chunk;              // tokens prepared into LDS at a time (what fits)
+  int H, G, dk, dv;
 };
 
-// LDS index of key channel i when a lane owns R consecutive channels: one float of
+// Everything of a token that does not depend on the state, for the delta rule: the unit
+// vectors, the decays and the write strengths, once per token instead of once per
+// workgroup that walks the token.  One workgroup a token.
+template <typename T>
+__global__ void __launch_bounds__(256)
+delta_prepare_kernel(const float* __restrict__ conv, int conv_width, int q_col, int k_col,
+                     const T* __restrict__ proj, int proj_stride, int gate_col,
+                     const T* __restrict__ decay, int decay_stride,
+                     const float* __restrict__ dt_bias, const float* __restrict__ A_log,
+                     float* __restrict__ prep, int prep_width, int H, int G, int dk) {
+  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float* row = prep + (size_t)t * prep_width;
+  for (int job = wave; job < 2 * G; job += 4) {
+    const int is_k = job >= G, g = is_k ? job - G : job;
+    const float* src = conv + (size_t)t * conv_width + (is_k ? k_col : q_col) + g * dk;
+    float ss = 0.f;
+    for (int i = lane; i < dk; i += 64) { const float v = src[i]; ss += v * v; }
+    ss = wave_sum(ss);
+    float scale = 1.0f / sqrtf(ss + 1e-6f);
+    if (!is_k) scale *= 1.0f / sqrtf((float)dk);
+    float* dst = row + (is_k ? G * dk : 0) + g * dk;
+    for (int i = lane; i < dk; i += 64) dst[i] = src[i] * scale;
+  }
+  for (int idx = tid; idx < H * dk; idx += 256) {
+    const float raw = to_f32<T>(decay[(size_t)t * decay_stride + idx]);
+    row[2 * G * dk + idx] = expf(-expf(A_log[idx / dk]) * softplus_f(raw + dt_bias[idx]));
+  }
+  for (int h = tid; h < H; h += 256)
+    row[2 * G * dk + H * dk + h] =
+        sigmoid_f(to_f32<T>(proj[(size_t)t * proj_stride + gate_col + h]));
+}
+
+#define RC_ROWS 16   // state rows a lane keeps
+
+// LDS index of key channel i when a lane owns RC_ROWS consecutive channels: one float of
 // padding per lane's share, so that the P lanes of a column meet different banks
-template <int R> __device__ __forceinline__ int lds_at(int i) { return i + i / R; }
+__device__ __forceinline__ int lds_at(int i) { return i + i / RC_ROWS; }
 
-template <typename T, int R, bool DELTA>
-__global__ void __launch_bounds__(512)
+// One wave a workgroup: 64 / P columns of one head's state, P lanes a column, RC_ROWS rows
+// a lane.  The vectors of the next CH tokens are requested into registers while the
+// current CH tokens are walked out of LDS, and put into the other LDS buffer afterwards.
+template <int P, bool DELTA>
+__global__ void __launch_bounds__(64, 2)
 matrix_recurrence_kernel(RecurrenceArgs a) {
-  extern __shared__ float lds[];
-  const int s = blockIdx.x, h = blockIdx.y;
-  const int tid = threadIdx.x;
-  const int P = a.P, dk = a.dk, dv = a.dv;
-  const int g = h / (a.H / a.G);
-  const int col = blockIdx.z * a.cols_per_block + tid / P, part = tid % P;
-  const bool owner = tid / P < a.cols_per_block && col < dv;
-  const int kpad = lds_at<R>(dk - 1) + 1;
-  // LDS: per chunk token: kvec[kpad], qvec[kpad], (delta) gvec[kpad], xvec[dv], 2 scalars
-  const int CH = a.chunk;
-  float* Kc = lds;
-  float* Qc = Kc + CH * kpad;
-  float* Gc = Qc + CH * kpad;
-  float* Xc = Gc + (DELTA ? CH * kpad : 0);
-  float* Sc = Xc + CH * dv;                // [chunk][2]: SSD (decay, dt); delta (beta, -)
+  constexpr int R = RC_ROWS;
+  constexpr int DKMAX = R * P;
+  constexpr int CH = P == 1 ? 16 : (P <= 8 ? 8 : (P == 16 ? 4 : (P == 32 ? 2 : 1)));
+  constexpr int NV = DELTA ? 3 : 2;                 // vectors of dk floats a token
+  constexpr int KPAD = DKMAX + P;                    // lds_at(DKMAX - 1) + 1
+  // a chunk's vectors come four floats a lane and load: LPV lanes cover a vector (or a
+  // quarter of a long one), so one load instruction of the wave brings TPL tokens' worth
+  constexpr int LPV = 4 * P < 64 ? 4 * P : 64;
+  constexpr int TPL = 64 / LPV;
+  constexpr int PIECES = DKMAX > 256 ? DKMAX / 256 : 1;
+  constexpr int NLOAD = NV * (CH / TPL) * PIECES;    // four-float loads a lane and chunk
+  __shared__ float vecs[2][CH][NV][KPAD];
+  __shared__ float scal[2][CH][2];                   // SSD: (decay, dt); delta: (beta, -)
 
+  const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int dk = a.dk, dv = a.dv;
+  const int g = h / (a.H / a.G);
+  const int col = blockIdx.z * (64 / P) + lane / P, part = lane % P;
+  const bool owner = col < dv;
   const int start = a.seq_start[s], n = a.seq_start[s + 1] - start;
-  float* st = a.state + (size_t)a.slot_id[s] * a.slot_stride + ((size_t)h * dv + col) * dk;
+
+  // where the token's vectors lie: vector v of token t starts at base[v] + t * stride
+  const float* base[NV];
+  int stride;
+  if (DELTA) {
+    stride = a.prep_width;
+    base[0] = a.prep + a.G * dk + g * dk;            // k
+    base[1] = a.prep + g * dk;                       // q
+    base[NV - 1] = a.prep + 2 * a.G * dk + h * dk;   // decays
+  } else {
+    stride = a.conv_width;
+    base[0] = a.conv + a.k_col + g * dk;
+    base[1] = a.conv + a.q_col + g * dk;
+  }
+  const float* xsrc = a.conv + a.x_col + h * dv + (owner ? col : 0);
+
+  float* st = a.state + (size_t)a.slot_id[s] * a.slot_stride + ((size_t)h * dv + col) * dk + part * R;
+  const bool vec_state = (dk % 4 == 0) && (a.slot_stride % 4 == 0) &&
+                         ((reinterpret_cast<uintptr_t>(a.state) & 15) == 0);
   float S[R];
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int i = part * R + r;
-    S[r] = (owner && i < dk) ? st[i] : 0.f;
-  }
-  const float neg_A = -expf(a.A_log[h]);
-  const float Dh = DELTA ? 0.f : a.D[h];
-  const int lane = tid & 63, wave = tid >> 6, nwaves = (blockDim.x + 63) >> 6;
-  const T* proj = (const T*)a.proj;
-  const T* decay = (const T*)a.decay;
-
-  for (int c0 = 0; c0 < n; c0 += CH) {
-    const int cn = n - c0 < CH ? n - c0 : CH;
-    __syncthreads();     // the chunk before has been walked
-    if (DELTA) {
-      // unit vectors: a wave takes (token, q or k) pairs in turn
-      for (int job = wave; job < 2 * cn; job += nwaves) {
-        const int tt = job >> 1, is_k = job & 1;
-        const float* src = a.conv + (size_t)(start + c0 + tt) * a.conv_width +
-                           (is_k ? a.k_col : a.q_col) + g * dk;
-        float ss = 0.f;
-        for (int i = lane; i < dk; i += 64) { const float v = src[i]; ss += v * v; }
-        ss = wave_sum(ss);
-        float scale = 1.0f / sqrtf(ss + 1e-6f);
-        if (!is_k) scale *= 1.0f / sqrtf((float)dk);
-        float* dst = (is_k ? Kc : Qc) + tt * kpad;
-        for (int i = lane; i < dk; i += 64) dst[lds_at<R>(i)] = src[i] * scale;
-      }
-      for (int idx = tid; idx < cn * dk; idx += blockDim.x) {
-        const int tt = idx / dk, i = idx % dk;
-        const float raw = to_f32<T>(decay[(size_t)(start + c0 + tt) * a.decay_stride + h * dk + i]);
-        Gc[tt * kpad + lds_at<R>(i)] = expf(neg_A * softplus_f(raw + a.dt_bias[h * dk + i]));
-      }
-      if (tid < cn)
-        Sc[tid * 2] = sigmoid_f(to_f32<T>(proj[(size_t)(start + c0 + tid) * a.proj_stride +
-                                               a.gate_col + h]));
+  for (int r = 0; r < R; ++r) S[r] = 0.f;
+  if (owner) {
+    if (vec_state) {
+#pragma unroll
+      for (int r = 0; r < R; r += 4)
+        if (part * R + r < dk) {
+          const float4 v = *reinterpret_cast<const float4*>(st + r);
+          S[r] = v.x; S[r + 1] = v.y; S[r + 2] = v.z; S[r + 3] = v.w;
+        }
     } else {
-      for (int idx = tid; idx < cn * dk; idx += blockDim.x) {
-        const int tt = idx / dk, i = idx % dk;
-        const float* row = a.conv + (size_t)(start + c0 + tt) * a.conv_width;
-        Kc[tt * kpad + lds_at<R>(i)] = row[a.k_col + g * dk + i];
-        Qc[tt * kpad + lds_at<R>(i)] = row[a.q_col + g * dk + i];
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        if (part * R + r < dk) S[r] = st[r];
+    }
+  }
+  const float neg_A = DELTA ? 0.f : -expf(a.A_log[h]);
+  const float Dh = DELTA ? 0.f : a.D[h];
+  const float dtb = DELTA ? 0.f : a.dt_bias[h];
+
+  // (whole four-float loads need the vectors to start on 16-byte boundaries)
+  bool vec_loads = dk % 4 == 0 && stride % 4 == 0;
+#pragma unroll
+  for (int v = 0; v < NV; ++v)
+    vec_loads = vec_loads && (reinterpret_cast<uintptr_t>(base[v]) & 15) == 0;
+  const int lane_tt = lane / LPV, lane_i = (lane % LPV) * 4;
+  float4 regs[NLOAD];
+  float xnext[CH], snext = 0.f;
+  auto request = [&](int c0) {
+#pragma unroll
+    for (int j = 0; j < NLOAD; ++j) {
+      const int v = j % NV, piece = (j / NV) % PIECES, group = j / (NV * PIECES);
+      const int tt = group * TPL + lane_tt, i = piece * 256 + lane_i;
+      float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (c0 + tt < n && i < dk) {
+        const float* src = base[v] + (size_t)(start + c0 + tt) * stride + i;
+        if (vec_loads) {
+          x = *reinterpret_cast<const float4*>(src);
+        } else {
+          x.x = src[0];
+          if (i + 1 < dk) x.y = src[1];
+          if (i + 2 < dk) x.z = src[2];
+          if (i + 3 < dk) x.w = src[3];
+        }
       }
-      if (tid < cn) {
-        const float raw = to_f32<T>(proj[(size_t)(start + c0 + tid) * a.proj_stride +
-                                         a.gate_col + h]);
-        const float dt = softplus_f(raw + a.dt_bias[h]);
-        Sc[tid * 2] = expf(neg_A * dt);
-        Sc[tid * 2 + 1] = dt;
+      regs[j] = x;
+    }
+#pragma unroll
+    for (int tt = 0; tt < CH; ++tt)
+      xnext[tt] = c0 + tt < n ? xsrc[(size_t)(start + c0 + tt) * a.conv_width] : 0.f;
+    if (lane < CH && c0 + lane < n) {
+      const size_t t = start + c0 + lane;
+      if (DELTA) {
+        snext = a.prep[t * a.prep_width + 2 * a.G * dk + a.H * dk + h];
+      } else {
+        const size_t at = t * a.proj_stride + a.gate_col + h;
+        snext = a.proj_bf16 ? (float)((const bf16_t*)a.proj)[at] : ((const float*)a.proj)[at];
       }
     }
-    for (int idx = tid; idx < cn * dv; idx += blockDim.x) {
-      const int tt = idx / dv, j = idx % dv;
-      Xc[tt * dv + j] = a.conv[(size_t)(start + c0 + tt) * a.conv_width + a.x_col + h * dv + j];
+  };
+  auto deposit = [&](int buf) {
+#pragma unroll
+    for (int j = 0; j < NLOAD; ++j) {
+      const int v = j % NV, piece = (j / NV) % PIECES, group = j / (NV * PIECES);
+      // (four channels from a multiple of four lie in one lane's share: side by side)
+      float* dst = &vecs[buf][group * TPL + lane_tt][v][lds_at(piece * 256 + lane_i)];
+      dst[0] = regs[j].x; dst[1] = regs[j].y; dst[2] = regs[j].z; dst[3] = regs[j].w;
+    }
+    if (lane < CH) {
+      if (DELTA) {
+        scal[buf][lane][0] = snext;
+      } else {
+        const float dt = softplus_f(snext + dtb);
+        scal[buf][lane][0] = expf(neg_A * dt);
+        scal[buf][lane][1] = dt;
+      }
+    }
+  };
+
+  float xcur[CH];
+  request(0);
+  deposit(0);
+#pragma unroll
+  for (int tt = 0; tt < CH; ++tt) xcur[tt] = xnext[tt];
+  __syncthreads();
+  for (int c0 = 0, buf = 0; c0 < n; c0 += CH, buf ^= 1) {
+    const bool more = c0 + CH < n;
+    if (more) request(c0 + CH);
+    const int cn = n - c0 < CH ? n - c0 : CH;
+#pragma unroll
+    for (int tt = 0; tt < CH; ++tt) {
+      if (tt < cn) {
+        const float* kk = &vecs[buf][tt][0][part * (R + 1)];
+        const float* qq = &vecs[buf][tt][1][part * (R + 1)];
+        const float xv = xcur[tt];
+        float o;
+        if (DELTA) {
+          const float* gg = &vecs[buf][tt][NV - 1][part * (R + 1)];
+          float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
+#pragma unroll
+          for (int r = 0; r < R; r += 4) {
+            S[r] *= gg[r]; S[r + 1] *= gg[r + 1]; S[r + 2] *= gg[r + 2]; S[r + 3] *= gg[r + 3];
+            d0 = fmaf(S[r], kk[r], d0);
+            d1 = fmaf(S[r + 1], kk[r + 1], d1);
+            d2 = fmaf(S[r + 2], kk[r + 2], d2);
+            d3 = fmaf(S[r + 3], kk[r + 3], d3);
+          }
+          float dot = (d0 + d1) + (d2 + d3);
+#pragma unroll
+          for (int off = 1; off < P; off <<= 1) dot += __shfl_xor(dot, off, ZA_WAVE);
+          const float u = scal[buf][tt][0] * (xv - dot);
+          float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+          for (int r = 0; r < R; r += 4) {
+            S[r] = fmaf(kk[r], u, S[r]);
+            S[r + 1] = fmaf(kk[r + 1], u, S[r + 1]);
+            S[r + 2] = fmaf(kk[r + 2], u, S[r + 2]);
+            S[r + 3] = fmaf(kk[r + 3], u, S[r + 3]);
+            a0 = fmaf(S[r], qq[r], a0);
+            a1 = fmaf(S[r + 1], qq[r + 1], a1);
+            a2 = fmaf(S[r + 2], qq[r + 2], a2);
+            a3 = fmaf(S[r + 3], qq[r + 3], a3);
+          }
+          float acc = (a0 + a1) + (a2 + a3);
+#pragma unroll
+          for (int off = 1; off < P; off <<= 1) acc += __shfl_xor(acc, off, ZA_WAVE);
+          o = acc;
+        } else {
+          const float decay_t = scal[buf][tt][0], dtx = scal[buf][tt][1] * xv;
+          float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+          for (int r = 0; r < R; r += 4) {
+            S[r] = fmaf(decay_t, S[r], dtx * kk[r]);
+            S[r + 1] = fmaf(decay_t, S[r + 1], dtx * kk[r + 1]);
+            S[r + 2] = fmaf(decay_t, S[r + 2], dtx * kk[r + 2]);
+            S[r + 3] = fmaf(decay_t, S[r + 3], dtx * kk[r + 3]);
+            a0 = fmaf(S[r], qq[r], a0);
+            a1 = fmaf(S[r + 1], qq[r + 1], a1);
+            a2 = fmaf(S[r + 2], qq[r + 2], a2);
+            a3 = fmaf(S[r + 3], qq[r + 3], a3);
+          }
+          float acc = (a0 + a1) + (a2 + a3);
+#pragma unroll
+          for (int off = 1; off < P; off <<= 1) acc += __shfl_xor(acc, off, ZA_WAVE);
+          o = fmaf(Dh, xv, acc);
+        }
+        if (part == 0 && owner)
+          a.out[(size_t)(start + c0 + tt) * a.H * dv + h * dv + col] = o;
+      }
+    }
+    if (more) {
+      deposit(buf ^ 1);
+#pragma unroll
+      for (int tt = 0; tt < CH; ++tt) xcur[tt] = xnext[tt];
     }
     __syncthreads();
-    if (!owner) continue;
-    for (int tt = 0; tt < cn; ++tt) {
-      const float* kk = Kc + tt * kpad + part * (R + 1);
-      const float* qq = Qc + tt * kpad + part * (R + 1);
-      const float xv = Xc[tt * dv + col];
-      float o;
-      if (DELTA) {
-        const float* gg = Gc + tt * kpad + part * (R + 1);
-        float dot = 0.f;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          if (part * R + r < dk) {
-            S[r] *= gg[r];
-            dot = fmaf(S[r], kk[r], dot);
-          }
-        }
-        for (int off = 1; off < P; off <<= 1) dot += __shfl_xor(dot, off, ZA_WAVE);
-        const float u = Sc[tt * 2] * (xv - dot);
-        float acc = 0.f;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          if (part * R + r < dk) {
-            S[r] = fmaf(kk[r], u, S[r]);
-            acc = fmaf(S[r], qq[r], acc);
-          }
-        }
-        for (int off = 1; off < P; off <<= 1) acc += __shfl_xor(acc, off, ZA_WAVE);
-        o = acc;
-      } else {
-        const float decay_t = Sc[tt * 2], dtx = Sc[tt * 2 + 1] * xv;
-        float acc = 0.f;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          if (part * R + r < dk) {
-            S[r] = fmaf(decay_t, S[r], dtx * kk[r]);
-            acc = fmaf(S[r], qq[r], acc);
-          }
-        }
-        for (int off = 1; off < P; off <<= 1) acc += __shfl_xor(acc, off, ZA_WAVE);
-        o = fmaf(Dh, xv, acc);
-      }
-      if (part == 0) a.out[(size_t)(start + c0 + tt) * a.H * dv + h * dv + col] = o;
-    }
   }
   if (owner) {
+    if (vec_state) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int i = part * R + r;
-      if (i < dk) st[i] = S[r];
+      for (int r = 0; r < R; r += 4)
+        if (part * R + r < dk)
+          *reinterpret_cast<float4*>(st + r) = make_float4(S[r], S[r + 1], S[r + 2], S[r + 3]);
+    } else {
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        if (part * R + r < dk) st[r] = S[r];
     }
   }
 }
 
-template <typename T, bool DELTA>
-static int launch_recurrence(RecurrenceArgs a, int n_seqs, int R, hipStream_t stream) {
-  const int threads = (a.cols_per_block * a.P + 63) / 64 * 64;
-  const int kpad = a.dk + (a.dk - 1) / R + 1;
-  const size_t per_token = sizeof(float) * ((size_t)kpad * (DELTA ? 3 : 2) + a.dv + 2);
-  a.chunk = RC_CHUNK;
-  while (a.chunk > 1 && a.chunk * per_token > 64 * 1024) a.chunk /= 2;
-  const size_t lds = a.chunk * per_token;
-  if (lds > 64 * 1024) return ZA_ERR_UNSUPPORTED;
-  dim3 grid(n_seqs, a.H, (a.dv + a.cols_per_block - 1) / a.cols_per_block), block(threads);
-#define ZA_RECURRENCE(RR)                                                                    \
-  hipLaunchKernelGGL((matrix_recurrence_kernel<T, RR, DELTA>), grid, block, lds, stream, a)
-  if (R == 8) ZA_RECURRENCE(8);
-  else if (R == 16) ZA_RECURRENCE(16);
-  else if (R == 32) ZA_RECURRENCE(32);
-  else return ZA_ERR_UNSUPPORTED;
+template <bool DELTA>
+static int launch_recurrence(const RecurrenceArgs& a, int n_seqs, int P, hipStream_t stream) {
+  dim3 grid(n_seqs, a.H, (a.dv * P + 63) / 64), block(64);
+#define ZA_RECURRENCE(PP)                                                                  \
+  case PP:                                                                                 \
+    hipLaunchKernelGGL((matrix_recurrence_kernel<PP, DELTA>), grid, block, 0, stream, a);  \
+    break
+  switch (P) {
+    ZA_RECURRENCE(1);
+    ZA_RECURRENCE(2);
+    ZA_RECURRENCE(4);
+    ZA_RECURRENCE(8);
+    ZA_RECURRENCE(16);
+    ZA_RECURRENCE(32);
+    ZA_RECURRENCE(64);
+    default: return ZA_ERR_UNSUPPORTED;
+  }
 #undef ZA_RECURRENCE
   return za_launch_status();
 }
 
-// `form`: 0 = SSD, 1 = gated delta rule.  `lanes` (P): a power of two up to 64 that
-// splits a column's dk rows; `rows_per_lane` (R): 8, 16 or 32 with R * P >= dk;
-// `cols_per_block` columns of S (times P lanes, at most 512 threads) a workgroup.
+// `form`: 0 = SSD, 1 = gated delta rule.  `lanes` (P): the power of two, at most 64, with
+// 16 * P >= dk that splits a column's rows.  `prep` (delta): [n_tokens][prep_width]
+// floats of scratch, prep_width >= 2*G*dk + H*dk + H.
 extern "C" int za_matrix_recurrence(int form, int dtype, const float* conv, int conv_width,
                                     int q_col, int k_col, int x_col, const void* proj,
                                     int proj_stride, int gate_col, const void* decay,
-                                    int decay_stride, const float* dt_bias, const float* A_log, const float* D,
-                                    float* state, long long slot_stride, const int* seq_start,
-                                    const int* slot_id, float* out, int n_seqs, int H, int G,
-                                    int dk, int dv, int lanes, int rows_per_lane,
-                                    int cols_per_block, hipStream_t stream) {
-  if (n_seqs == 0) return 0;
-  if (n_seqs < 0 || H <= 0 || G <= 0 || H % G || dk <= 0 || dv <= 0 || !conv || !proj ||
-      !dt_bias || !A_log || !state || !seq_start || !slot_id || !out)
+                                    int decay_stride, const float* dt_bias, const float* A_log,
+                                    const float* D, float* prep, int prep_width, float* state,
+                                    long long slot_stride, const int* seq_start,
+                                    const int* slot_id, float* out, int n_tokens, int n_seqs,
+                                    int H, int G, int dk, int dv, int lanes,
+                                    hipStream_t stream) {
+  if (n_seqs == 0 || n_tokens == 0) return 0;
+  if (n_seqs < 0 || n_tokens < 0 || H <= 0 || G <= 0 || H % G || dk <= 0 || dv <= 0 || !conv ||
+      !proj || !dt_bias || !A_log || !state || !seq_start || !slot_id || !out)
     return ZA_ERR_ARG;
-  if (form == 0 ? !D : (!decay || decay_stride < H * dk)) return ZA_ERR_ARG;
-  if (lanes < 1 || lanes > 64 || (lanes & (lanes - 1)) || lanes * rows_per_lane < dk ||
-      cols_per_block < 1 || cols_per_block * lanes > 512 ||
+  if (form == 0 ? !D : (!decay || decay_stride < H * dk || !prep ||
+                        prep_width < 2 * G * dk + H * dk + H))
+    return ZA_ERR_ARG;
+  if (lanes < 1 || lanes > 64 || (lanes & (lanes - 1)) || lanes * RC_ROWS < dk ||
       slot_stride < (long long)H * dk * dv)
     return ZA_ERR_ARG;
-  RecurrenceArgs a{conv, conv_width, q_col, k_col, x_col, proj, proj_stride, gate_col, decay,
-                   decay_stride, dt_bias, A_log, D, state, slot_stride, seq_start, slot_id, out,
-                   H, G, dk, dv, lanes, cols_per_block, RC_CHUNK};
+  if (dtype != 0 && dtype != 1) return ZA_ERR_UNSUPPORTED;
+  RecurrenceArgs a{conv, conv_width, q_col, k_col, x_col, proj, proj_stride, gate_col, dtype,
+                   prep, prep_width, dt_bias, A_log, D, state, slot_stride, seq_start, slot_id,
+                   out, H, G, dk, dv};
+  if (form == 0) return launch_recurrence<false>(a, n_seqs, lanes, stream);
   if (dtype == 0)
-    return form ? launch_recurrence<float, true>(a, n_seqs, rows_per_lane, stream)
-                : launch_recurrence<float, false>(a, n_seqs, rows_per_lane, stream);
-  if (dtype == 1)
-    return form ? launch_recurrence<bf16_t, true>(a, n_seqs, rows_per_lane, stream)
-                : launch_recurrence<bf16_t, false>(a, n_seqs, rows_per_lane, stream);
-  return ZA_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL((delta_prepare_kernel<float>), dim3(n_tokens), dim3(256), 0, stream, conv,
+                       conv_width, q_col, k_col, (const float*)proj, proj_stride, gate_col,
+                       (const float*)decay, decay_stride, dt_bias, A_log, prep, prep_width, H, G,
+                       dk);
+  else
+    hipLaunchKernelGGL((delta_prepare_kernel<bf16_t>), dim3(n_tokens), dim3(256), 0, stream, conv,
+                       conv_width, q_col, k_col, (const bf16_t*)proj, proj_stride, gate_col,
+                       (const bf16_t*)decay, decay_stride, dt_bias, A_log, prep, prep_width, H, G,
+                       dk);
+  const int rc = za_launch_status();
+  if (rc != 0) return rc;
+  return launch_recurrence<true>(a, n_seqs, lanes, stream);
 }
 
 // ------------------------------------------------------------- gated group norm

@@ -105,10 +105,10 @@ _SIGNATURES = {
                                            c_void_p, c_longlong, c_void_p, c_void_p, c_void_p,
                                            c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     ("recurrent", "za_matrix_recurrence"): [c_int, c_int, c_void_p, c_int, c_int, c_int, c_int,
-                                            c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p,
-                                            c_void_p, c_void_p, c_longlong, c_void_p, c_void_p,
-                                            c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                                            c_int, c_int, c_void_p],
+                                            c_void_p, c_int, c_int, c_void_p, c_int, c_void_p,
+                                            c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                            c_longlong, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                            c_int, c_int, c_int, c_int, c_int, c_void_p],
     ("recurrent", "za_gated_group_norm"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int,
                                            c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
                                            c_int, c_int, c_float, c_void_p],
@@ -1591,17 +1591,18 @@ def causal_conv_silu(x: torch.Tensor, col0: int, taps: torch.Tensor, bias: Optio
     return out
 
 
+RECURRENCE_ROWS_PER_LANE = 16
+
+
 def recurrence_plan(dk: int, dv: int) -> Tuple[int, int, int]:
     """(lanes that split a column's rows, rows per lane, columns per workgroup) for a
-    state of ``dk`` rows and ``dv`` columns."""
+    state of ``dk`` rows and ``dv`` columns: a workgroup is one wave."""
     lanes = 1
-    while lanes * 16 < dk:
+    while lanes * RECURRENCE_ROWS_PER_LANE < dk:
         lanes *= 2
     if lanes > 64:
         raise KernelError(f"a state of {dk} rows exceeds the recurrence kernel's limit of 1024")
-    rows = 8 if lanes * 8 >= dk else 16
-    cols = max(1, min(dv, 256 // lanes))
-    return lanes, rows, cols
+    return lanes, RECURRENCE_ROWS_PER_LANE, 64 // lanes
 
 
 def matrix_recurrence(form: str, conv: torch.Tensor, q_col: int, k_col: int, x_col: int,
@@ -1645,14 +1646,19 @@ def matrix_recurrence(form: str, conv: torch.Tensor, q_col: int, k_col: int, x_c
     _need(seq_start, "seq_start", torch.int32, (S + 1,))
     _need(slot_id, "slot_id", torch.int32, (S,))
     base, slot_stride = _state_window(state, state_offset, heads * dk * dv, "state")
-    lanes, rows, cols = recurrence_plan(dk, dv)
+    lanes, _, _ = recurrence_plan(dk, dv)
     out = torch.empty((T, heads * dv), dtype=torch.float32, device=conv.device)
+    prep, prep_width = None, 0
+    if delta:
+        # what a token brings that does not depend on the state: unit q and k, decays, betas
+        prep_width = -(-(2 * groups * dk + heads * dk + heads) // 4) * 4
+        prep = torch.empty((T, prep_width), dtype=torch.float32, device=conv.device)
     rc = _fn("recurrent", "za_matrix_recurrence")(
         1 if delta else 0, _code(proj.dtype), _ptr(conv), conv_width, int(q_col), int(k_col),
         int(x_col), _ptr(proj), proj.shape[1], int(gate_col), _ptr(decay) if delta else None,
-        decay.shape[1] if delta else 0, _ptr(dt_bias), _ptr(A_log), None if delta else _ptr(D), base, slot_stride,
-        _ptr(seq_start), _ptr(slot_id), _ptr(out), S, heads, groups, dk, dv, lanes, rows, cols,
-        _stream())
+        decay.shape[1] if delta else 0, _ptr(dt_bias), _ptr(A_log), None if delta else _ptr(D),
+        _ptr(prep), prep_width, base, slot_stride, _ptr(seq_start), _ptr(slot_id), _ptr(out), T,
+        S, heads, groups, dk, dv, lanes, _stream())
     _check(rc, "matrix_recurrence", f"form={form} heads={heads} dk={dk} dv={dv}")
     return out
 

@@ -302,8 +302,8 @@ class GroupedQueryAttention(Mixer):
         if getattr(step, "taps", None) is not None:
             step.taps["q"] = q.clone()
             step.taps["o"] = o.clone()
-        return ops.linear(o.view(T, nh * dv), self.w_out, self.b_out, partial_ok=True,
-                          accumulate=stream, tune=self.runtime.tune)
+        return ops.linear(o.view(T, nh * dv), self.w_out, self.b_out, accumulate=stream,
+                          tune=self.runtime.tune)
 
     def _leave_taps(self, step, cache, q: torch.Tensor, o: torch.Tensor) -> None:
         """Diagnostics: the queries, the keys and values of the step's tokens as they lie in
