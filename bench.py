@@ -186,6 +186,29 @@ def compare(widths, layers, batch, prompt_len, steps, warmup) -> dict:
         torch.cuda.synchronize()
         seconds = (time.perf_counter() - t0) / 6
         out["prefill"] = {"tokens": prompt_len, "ms": seconds * 1e3, "tokens_per_s": prompt_len / seconds}
+        # ---- the same number of tokens as eight prompts in one step (what a server's
+        # steps look like): a layer that walks its tokens in order walks an eighth as many
+        part = prompt_len // 8
+
+        def eight(tag):
+            names = [(tag, i) for i in range(8)]
+            for name in names:
+                runner.admit(name)
+            runner.step([StepEntry(name, tokens(part), [part - 1]) for name in names])
+            for name in names:
+                runner.release(name)
+        del runner
+        runner = ModelRunner(model, page_size=page, num_pages=8 * (part // page + 2), num_slots=8)
+        for r in range(3):
+            eight(("w8", r))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for r in range(6):
+            eight(("p8", r))
+        torch.cuda.synchronize()
+        seconds = (time.perf_counter() - t0) / 6
+        out["prefill_8_prompts"] = {"tokens": 8 * part, "ms": seconds * 1e3,
+                                    "tokens_per_s": 8 * part / seconds}
         del runner
         torch.cuda.empty_cache()
         # ---- decode: a batch at that context, steps issued as generation issues them

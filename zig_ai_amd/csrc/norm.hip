@@ -228,6 +228,7 @@ extern "C" int za_embed_gather(const int* tokens, const void* table, int table_d
 //   x <- x + sa * a + sb * b      (b may be absent; 32-bit sum, stored)
 //   out = x / sqrt(mean(x^2) + eps) * weight      (when a norm's weight is given)
 // `a` and `b` are in the storage type TD.  One workgroup a row, two passes.
+#define SA_VPT 16   // values a thread keeps between the sum of squares and the scaling
 template <typename TD, typename TO>
 __global__ void __launch_bounds__(256)
 scaled_add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ a, float sa,
@@ -238,8 +239,40 @@ scaled_add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ a
   float* x = residual + r * width;
   const TD* ar = a + r * width;
   const TD* br = b ? b + r * width : nullptr;
+  const int bd = blockDim.x;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+  if (width <= bd * SA_VPT) {
+    // the row stays in registers: one trip to memory, every load requested at once
+    float h[SA_VPT], wv[SA_VPT];
+#pragma unroll
+    for (int k = 0; k < SA_VPT; ++k) {
+      const int i = threadIdx.x + k * bd;
+      const bool in = i < width;
+      h[k] = in ? x[i] : 0.f;
+      const float av = in ? to_f32<TD>(ar[i]) : 0.f;
+      const float bv = (in && br) ? to_f32<TD>(br[i]) : 0.f;
+      wv[k] = (in && weight) ? weight[i] : 0.f;
+      h[k] = fmaf(sa, av, h[k]);
+      if (br) h[k] = fmaf(sb, bv, h[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < SA_VPT; ++k) {
+      const int i = threadIdx.x + k * bd;
+      if (i < width) x[i] = h[k];
+      ss += h[k] * h[k];
+    }
+    if (!weight) return;
+    ss = block_sum(ss, scratch);
+    const float scale = 1.0f / sqrtf(ss / (float)width + eps);
+    TO* o = out + r * width;
+#pragma unroll
+    for (int k = 0; k < SA_VPT; ++k) {
+      const int i = threadIdx.x + k * bd;
+      if (i < width) o[i] = from_f32<TO>(h[k] * scale * wv[k]);
+    }
+    return;
+  }
+  for (int i = threadIdx.x; i < width; i += bd) {
     float h = fmaf(sa, to_f32<TD>(ar[i]), x[i]);
     if (br) h = fmaf(sb, to_f32<TD>(br[i]), h);
     x[i] = h;
@@ -249,7 +282,7 @@ scaled_add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ a
   ss = block_sum(ss, scratch);
   const float scale = 1.0f / sqrtf(ss / (float)width + eps);
   TO* o = out + r * width;
-  for (int i = threadIdx.x; i < width; i += blockDim.x)
+  for (int i = threadIdx.x; i < width; i += bd)
     o[i] = from_f32<TO>(x[i] * scale * weight[i]);   // this thread stored x[i] above
 }
 

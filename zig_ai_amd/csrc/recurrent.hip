@@ -161,17 +161,19 @@ struct RecurrenceArgs {
 
 // Everything of a token that does not depend on the state, for the delta rule: the unit
 // vectors, the decays and the write strengths, once per token instead of once per
-// workgroup that walks the token.  One workgroup a token.
+// workgroup that walks the token.  grid (tokens, jobs): the first 2*G jobs of a token make
+// one unit vector each, the others take 256 decays each, the last one also the betas; a
+// job is one trip to memory, and the jobs of a token run side by side.
 template <typename T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(64)
 delta_prepare_kernel(const float* __restrict__ conv, int conv_width, int q_col, int k_col,
                      const T* __restrict__ proj, int proj_stride, int gate_col,
                      const T* __restrict__ decay, int decay_stride,
                      const float* __restrict__ dt_bias, const float* __restrict__ A_log,
                      float* __restrict__ prep, int prep_width, int H, int G, int dk) {
-  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int t = blockIdx.x, job = blockIdx.y, lane = threadIdx.x;
   float* row = prep + (size_t)t * prep_width;
-  for (int job = wave; job < 2 * G; job += 4) {
+  if (job < 2 * G) {
     const int is_k = job >= G, g = is_k ? job - G : job;
     const float* src = conv + (size_t)t * conv_width + (is_k ? k_col : q_col) + g * dk;
     float ss = 0.f;
@@ -181,14 +183,21 @@ delta_prepare_kernel(const float* __restrict__ conv, int conv_width, int q_col, 
     if (!is_k) scale *= 1.0f / sqrtf((float)dk);
     float* dst = row + (is_k ? G * dk : 0) + g * dk;
     for (int i = lane; i < dk; i += 64) dst[i] = src[i] * scale;
+    return;
   }
-  for (int idx = tid; idx < H * dk; idx += 256) {
-    const float raw = to_f32<T>(decay[(size_t)t * decay_stride + idx]);
-    row[2 * G * dk + idx] = expf(-expf(A_log[idx / dk]) * softplus_f(raw + dt_bias[idx]));
+  const int first = (job - 2 * G) * 256;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int idx = first + lane + 64 * k;
+    if (idx < H * dk) {
+      const float raw = to_f32<T>(decay[(size_t)t * decay_stride + idx]);
+      row[2 * G * dk + idx] = expf(-expf(A_log[idx / dk]) * softplus_f(raw + dt_bias[idx]));
+    }
   }
-  for (int h = tid; h < H; h += 256)
-    row[2 * G * dk + H * dk + h] =
-        sigmoid_f(to_f32<T>(proj[(size_t)t * proj_stride + gate_col + h]));
+  if (job == (int)gridDim.y - 1)
+    for (int h = lane; h < H; h += 64)
+      row[2 * G * dk + H * dk + h] =
+          sigmoid_f(to_f32<T>(proj[(size_t)t * proj_stride + gate_col + h]));
 }
 
 #define RC_ROWS 16   // state rows a lane keeps
@@ -197,15 +206,41 @@ delta_prepare_kernel(const float* __restrict__ conv, int conv_width, int q_col, 
 // padding per lane's share, so that the P lanes of a column meet different banks
 __device__ __forceinline__ int lds_at(int i) { return i + i / RC_ROWS; }
 
+// The sum over the P neighbouring lanes (a power of two, the group starting at a multiple
+// of P) that share a column; every lane of the group gets it.  Up to sixteen lanes the
+// partners are reached with the vector unit's own lane patterns (pairs, quads, a half
+// row and a row of sixteen mirrored), beyond that through the lane exchange.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float x) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, false);
+  return x + __builtin_bit_cast(float, moved);
+}
+
+template <int P>
+__device__ __forceinline__ float group_sum(float x) {
+  if (P >= 2) x = dpp_add<0xB1>(x);     // lanes 1 0 3 2 of every four
+  if (P >= 4) x = dpp_add<0x4E>(x);     // lanes 2 3 0 1 of every four
+  if (P >= 8) x = dpp_add<0x141>(x);    // a half row of eight, mirrored
+  if (P >= 16) x = dpp_add<0x140>(x);   // a row of sixteen, mirrored
+  if (P >= 32) x += __shfl_xor(x, 16, ZA_WAVE);
+  if (P >= 64) x += __shfl_xor(x, 32, ZA_WAVE);
+  return x;
+}
+
 // One wave a workgroup: 64 / P columns of one head's state, P lanes a column, RC_ROWS rows
 // a lane.  The vectors of the next CH tokens are requested into registers while the
 // current CH tokens are walked out of LDS, and put into the other LDS buffer afterwards.
-template <int P, bool DELTA>
+// LONG: portions of many tokens (chunks of up to sixteen tokens, so that a chunk's walk
+// outlasts the trip to memory of the next one's vectors); otherwise chunks as short as the
+// load pattern allows, which leaves LDS for more waves when every portion is a token or two.
+template <int P, bool DELTA, bool LONG>
 __global__ void __launch_bounds__(64, 2)
 matrix_recurrence_kernel(RecurrenceArgs a) {
   constexpr int R = RC_ROWS;
   constexpr int DKMAX = R * P;
-  constexpr int CH = P == 1 ? 16 : (P <= 8 ? 8 : (P == 16 ? 4 : (P == 32 ? 2 : 1)));
+  constexpr int CH_MIN = 4 * P < 64 ? 64 / (4 * P) : 1;
+  constexpr int CH_LONG = P <= 8 ? 16 : (P == 16 ? 8 : (P == 32 ? 4 : 2));
+  constexpr int CH = LONG ? CH_LONG : (CH_MIN < 2 ? 2 : CH_MIN);
   constexpr int NV = DELTA ? 3 : 2;                 // vectors of dk floats a token
   constexpr int KPAD = DKMAX + P;                    // lds_at(DKMAX - 1) + 1
   // a chunk's vectors come four floats a lane and load: LPV lanes cover a vector (or a
@@ -332,8 +367,11 @@ matrix_recurrence_kernel(RecurrenceArgs a) {
     const bool more = c0 + CH < n;
     if (more) request(c0 + CH);
     const int cn = n - c0 < CH ? n - c0 : CH;
+    float result[CH];      // stored after the walk: a store among the requests would make
+                           // the walk wait for everything requested before it
 #pragma unroll
     for (int tt = 0; tt < CH; ++tt) {
+      result[tt] = 0.f;
       if (tt < cn) {
         const float* kk = &vecs[buf][tt][0][part * (R + 1)];
         const float* qq = &vecs[buf][tt][1][part * (R + 1)];
@@ -350,9 +388,7 @@ matrix_recurrence_kernel(RecurrenceArgs a) {
             d2 = fmaf(S[r + 2], kk[r + 2], d2);
             d3 = fmaf(S[r + 3], kk[r + 3], d3);
           }
-          float dot = (d0 + d1) + (d2 + d3);
-#pragma unroll
-          for (int off = 1; off < P; off <<= 1) dot += __shfl_xor(dot, off, ZA_WAVE);
+          const float dot = group_sum<P>((d0 + d1) + (d2 + d3));
           const float u = scal[buf][tt][0] * (xv - dot);
           float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
 #pragma unroll
@@ -366,10 +402,7 @@ matrix_recurrence_kernel(RecurrenceArgs a) {
             a2 = fmaf(S[r + 2], qq[r + 2], a2);
             a3 = fmaf(S[r + 3], qq[r + 3], a3);
           }
-          float acc = (a0 + a1) + (a2 + a3);
-#pragma unroll
-          for (int off = 1; off < P; off <<= 1) acc += __shfl_xor(acc, off, ZA_WAVE);
-          o = acc;
+          o = group_sum<P>((a0 + a1) + (a2 + a3));
         } else {
           const float decay_t = scal[buf][tt][0], dtx = scal[buf][tt][1] * xv;
           float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
@@ -384,14 +417,15 @@ matrix_recurrence_kernel(RecurrenceArgs a) {
             a2 = fmaf(S[r + 2], qq[r + 2], a2);
             a3 = fmaf(S[r + 3], qq[r + 3], a3);
           }
-          float acc = (a0 + a1) + (a2 + a3);
-#pragma unroll
-          for (int off = 1; off < P; off <<= 1) acc += __shfl_xor(acc, off, ZA_WAVE);
-          o = fmaf(Dh, xv, acc);
+          o = fmaf(Dh, xv, group_sum<P>((a0 + a1) + (a2 + a3)));
         }
-        if (part == 0 && owner)
-          a.out[(size_t)(start + c0 + tt) * a.H * dv + h * dv + col] = o;
+        result[tt] = o;
       }
+    }
+    if (part == 0 && owner) {
+#pragma unroll
+      for (int tt = 0; tt < CH; ++tt)
+        if (tt < cn) a.out[(size_t)(start + c0 + tt) * a.H * dv + h * dv + col] = result[tt];
     }
     if (more) {
       deposit(buf ^ 1);
@@ -415,11 +449,15 @@ matrix_recurrence_kernel(RecurrenceArgs a) {
 }
 
 template <bool DELTA>
-static int launch_recurrence(const RecurrenceArgs& a, int n_seqs, int P, hipStream_t stream) {
+static int launch_recurrence(const RecurrenceArgs& a, int n_seqs, int P, bool long_portions,
+                             hipStream_t stream) {
   dim3 grid(n_seqs, a.H, (a.dv * P + 63) / 64), block(64);
-#define ZA_RECURRENCE(PP)                                                                  \
-  case PP:                                                                                 \
-    hipLaunchKernelGGL((matrix_recurrence_kernel<PP, DELTA>), grid, block, 0, stream, a);  \
+#define ZA_RECURRENCE(PP)                                                                      \
+  case PP:                                                                                     \
+    if (long_portions)                                                                         \
+      hipLaunchKernelGGL((matrix_recurrence_kernel<PP, DELTA, true>), grid, block, 0, stream, a);  \
+    else                                                                                       \
+      hipLaunchKernelGGL((matrix_recurrence_kernel<PP, DELTA, false>), grid, block, 0, stream, a); \
     break
   switch (P) {
     ZA_RECURRENCE(1);
@@ -461,24 +499,28 @@ extern "C" int za_matrix_recurrence(int form, int dtype, const float* conv, int 
   RecurrenceArgs a{conv, conv_width, q_col, k_col, x_col, proj, proj_stride, gate_col, dtype,
                    prep, prep_width, dt_bias, A_log, D, state, slot_stride, seq_start, slot_id,
                    out, H, G, dk, dv};
-  if (form == 0) return launch_recurrence<false>(a, n_seqs, lanes, stream);
+  // (a function of the step's shape alone, as a recorded step needs it)
+  const bool long_portions = n_tokens > 4 * n_seqs;
+  if (form == 0) return launch_recurrence<false>(a, n_seqs, lanes, long_portions, stream);
+  const dim3 prep_grid(n_tokens, 2 * G + (H * dk + 255) / 256);
   if (dtype == 0)
-    hipLaunchKernelGGL((delta_prepare_kernel<float>), dim3(n_tokens), dim3(256), 0, stream, conv,
+    hipLaunchKernelGGL((delta_prepare_kernel<float>), prep_grid, dim3(64), 0, stream, conv,
                        conv_width, q_col, k_col, (const float*)proj, proj_stride, gate_col,
                        (const float*)decay, decay_stride, dt_bias, A_log, prep, prep_width, H, G,
                        dk);
   else
-    hipLaunchKernelGGL((delta_prepare_kernel<bf16_t>), dim3(n_tokens), dim3(256), 0, stream, conv,
+    hipLaunchKernelGGL((delta_prepare_kernel<bf16_t>), prep_grid, dim3(64), 0, stream, conv,
                        conv_width, q_col, k_col, (const bf16_t*)proj, proj_stride, gate_col,
                        (const bf16_t*)decay, decay_stride, dt_bias, A_log, prep, prep_width, H, G,
                        dk);
   const int rc = za_launch_status();
   if (rc != 0) return rc;
-  return launch_recurrence<true>(a, n_seqs, lanes, stream);
+  return launch_recurrence<true>(a, n_seqs, lanes, long_portions, stream);
 }
 
 // ------------------------------------------------------------- gated group norm
 // grid (tokens, groups); a workgroup reduces one group of `group` columns.
+#define GN_VPT 16   // values a thread keeps between the sum of squares and the scaling
 template <typename T>
 __global__ void __launch_bounds__(256)
 gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ gate, int gate_stride,
@@ -489,8 +531,37 @@ gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ gate,
   const int t = blockIdx.x, c0 = blockIdx.y * group;
   const float* yr = y + (size_t)t * width + c0;
   const T* gr = gate + (size_t)t * gate_stride + gate_col + c0;
+  T* o = out + (size_t)t * out_stride + out_col + c0;
+  const int bd = blockDim.x;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < group; i += blockDim.x) {
+  if (group <= bd * GN_VPT) {
+    // one trip to memory: every load is requested before anything is summed
+    float v[GN_VPT], act[GN_VPT], wv[GN_VPT];
+#pragma unroll
+    for (int k = 0; k < GN_VPT; ++k) {
+      const int i = threadIdx.x + k * bd;
+      v[k] = i < group ? yr[i] : 0.f;
+      act[k] = i < group ? to_f32<T>(gr[i]) : 0.f;
+      wv[k] = i < group ? w[(c0 + i) % wlen] : 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < GN_VPT; ++k) {
+      act[k] = silu_gate ? silu_f(act[k]) : sigmoid_f(act[k]);
+      if (gate_first) v[k] *= act[k];
+      ss += v[k] * v[k];
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = 1.0f / sqrtf(ss / (float)group + eps);
+#pragma unroll
+    for (int k = 0; k < GN_VPT; ++k) {
+      const int i = threadIdx.x + k * bd;
+      float r = v[k] * scale * wv[k];
+      if (!gate_first) r *= act[k];
+      if (i < group) o[i] = from_f32<T>(r * out_scale);
+    }
+    return;
+  }
+  for (int i = threadIdx.x; i < group; i += bd) {
     float v = yr[i];
     if (gate_first) {
       const float gv = to_f32<T>(gr[i]);
@@ -500,8 +571,7 @@ gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ gate,
   }
   ss = block_sum(ss, scratch);
   const float scale = 1.0f / sqrtf(ss / (float)group + eps);
-  T* o = out + (size_t)t * out_stride + out_col + c0;
-  for (int i = threadIdx.x; i < group; i += blockDim.x) {
+  for (int i = threadIdx.x; i < group; i += bd) {
     const float gv = to_f32<T>(gr[i]);
     const float act = silu_gate ? silu_f(gv) : sigmoid_f(gv);
     float v = yr[i];

@@ -90,7 +90,15 @@ class ScaledResidualBlock:
     def forward(self, residual: torch.Tensor, pending: Optional[torch.Tensor], step,
                 cache) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
         from ..kernels import ops
-        h = self.mixer_norm.add_forward(residual, pending)
+        h = None
+        if pending is None and all(getattr(p, "takes_stream", False)
+                                   or getattr(p, "takes_normed_rows", False)
+                                   for p in self.mixer_parts):
+            # a decode batch: the mixers' opening products run the norm themselves (the
+            # stream is added to only after every mixer has returned)
+            h = self.mixer_norm.deferred(residual)
+        if h is None:
+            h = self.mixer_norm.add_forward(residual, pending)
         if len(self.mixers) == 1:
             outs = [self.mixer_parts[0].forward(h, step, cache)]
         else:
@@ -103,7 +111,7 @@ class ScaledResidualBlock:
         norm = self.feed_forward_norm
         if hasattr(norm, "weight") and hasattr(norm, "eps"):
             h = ops.scaled_add_rmsnorm(residual, outs[0], self.mixer_scales[0], *second,
-                                       weight=norm.weight, eps=norm.eps, out_dtype=h.dtype)
+                                       weight=norm.weight, eps=norm.eps, out_dtype=outs[0].dtype)
         else:
             ops.scaled_add_rmsnorm(residual, outs[0], self.mixer_scales[0], *second)
             h = norm.forward(residual)

@@ -39,6 +39,7 @@ from .feed_forward import fuse_rows, pad_columns, pad_rows
 class StateSpaceDuality(Mixer):
     kind = "ssd"
     graph_safe = True
+    takes_normed_rows = True      # ``x`` is only ever handed to ``ops.linear``
     kernel_sources = ("gemm", "recurrent")
 
     @staticmethod
@@ -107,6 +108,7 @@ class StateSpaceDuality(Mixer):
 class GatedDeltaRule(Mixer):
     kind = "gated_delta"
     graph_safe = True
+    takes_normed_rows = True      # ``x`` is only ever handed to ``ops.linear``
     kernel_sources = ("gemm", "recurrent", "activation")
 
     @staticmethod
