@@ -202,9 +202,12 @@ delta_prepare_kernel(const float* __restrict__ conv, int conv_width, int q_col, 
 
 #define RC_ROWS 16   // state rows a lane keeps
 
-// LDS index of key channel i when a lane owns RC_ROWS consecutive channels: one float of
-// padding per lane's share, so that the P lanes of a column meet different banks
-__device__ __forceinline__ int lds_at(int i) { return i + i / RC_ROWS; }
+// LDS index of key channel i when a lane owns RC_ROWS consecutive channels: four floats of
+// padding per lane's share, so that a share starts on a 16-byte boundary (four-float
+// reads) and the eight shares that eight neighbouring lanes read at once, 20 floats
+// apart, cover the 32 banks once
+#define RC_SHARE (RC_ROWS + 4)
+__device__ __forceinline__ int lds_at(int i) { return i + (i / RC_ROWS) * 4; }
 
 // The sum over the P neighbouring lanes (a power of two, the group starting at a multiple
 // of P) that share a column; every lane of the group gets it.  Up to sixteen lanes the
@@ -233,23 +236,25 @@ __device__ __forceinline__ float group_sum(float x) {
 // LONG: portions of many tokens (chunks of up to sixteen tokens, so that a chunk's walk
 // outlasts the trip to memory of the next one's vectors); otherwise chunks as short as the
 // load pattern allows, which leaves LDS for more waves when every portion is a token or two.
-template <int P, bool DELTA, bool LONG>
+// (LONG == 1: half as long chunks, for steps with more waves than the chip has SIMDs, where
+// LDS decides how many of them run at once)
+template <int P, bool DELTA, int LONG>
 __global__ void __launch_bounds__(64, 2)
 matrix_recurrence_kernel(RecurrenceArgs a) {
   constexpr int R = RC_ROWS;
   constexpr int DKMAX = R * P;
   constexpr int CH_MIN = 4 * P < 64 ? 64 / (4 * P) : 1;
-  constexpr int CH_LONG = P <= 8 ? 16 : (P == 16 ? 8 : (P == 32 ? 4 : 2));
-  constexpr int CH = LONG ? CH_LONG : (CH_MIN < 2 ? 2 : CH_MIN);
+  constexpr int CH_LONG = (P <= 8 ? 16 : (P == 16 ? 8 : (P == 32 ? 4 : 2))) / (LONG == 1 ? 2 : 1);
+  constexpr int CH = LONG ? (CH_LONG < CH_MIN ? CH_MIN : CH_LONG) : (CH_MIN < 2 ? 2 : CH_MIN);
   constexpr int NV = DELTA ? 3 : 2;                 // vectors of dk floats a token
-  constexpr int KPAD = DKMAX + P;                    // lds_at(DKMAX - 1) + 1
+  constexpr int KPAD = RC_SHARE * P;
   // a chunk's vectors come four floats a lane and load: LPV lanes cover a vector (or a
   // quarter of a long one), so one load instruction of the wave brings TPL tokens' worth
   constexpr int LPV = 4 * P < 64 ? 4 * P : 64;
   constexpr int TPL = 64 / LPV;
   constexpr int PIECES = DKMAX > 256 ? DKMAX / 256 : 1;
   constexpr int NLOAD = NV * (CH / TPL) * PIECES;    // four-float loads a lane and chunk
-  __shared__ float vecs[2][CH][NV][KPAD];
+  __shared__ __attribute__((aligned(16))) float vecs[2][CH][NV][KPAD];
   __shared__ float scal[2][CH][2];                   // SSD: (decay, dt); delta: (beta, -)
 
   const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -343,8 +348,8 @@ matrix_recurrence_kernel(RecurrenceArgs a) {
     for (int j = 0; j < NLOAD; ++j) {
       const int v = j % NV, piece = (j / NV) % PIECES, group = j / (NV * PIECES);
       // (four channels from a multiple of four lie in one lane's share: side by side)
-      float* dst = &vecs[buf][group * TPL + lane_tt][v][lds_at(piece * 256 + lane_i)];
-      dst[0] = regs[j].x; dst[1] = regs[j].y; dst[2] = regs[j].z; dst[3] = regs[j].w;
+      *reinterpret_cast<float4*>(&vecs[buf][group * TPL + lane_tt][v][lds_at(piece * 256 + lane_i)]) =
+          regs[j];
     }
     if (lane < CH) {
       if (DELTA) {
@@ -373,12 +378,24 @@ matrix_recurrence_kernel(RecurrenceArgs a) {
     for (int tt = 0; tt < CH; ++tt) {
       result[tt] = 0.f;
       if (tt < cn) {
-        const float* kk = &vecs[buf][tt][0][part * (R + 1)];
-        const float* qq = &vecs[buf][tt][1][part * (R + 1)];
+        float kk[R], qq[R];
+#pragma unroll
+        for (int r = 0; r < R; r += 4) {
+          const float4 k4 = *reinterpret_cast<const float4*>(&vecs[buf][tt][0][part * RC_SHARE + r]);
+          const float4 q4 = *reinterpret_cast<const float4*>(&vecs[buf][tt][1][part * RC_SHARE + r]);
+          kk[r] = k4.x; kk[r + 1] = k4.y; kk[r + 2] = k4.z; kk[r + 3] = k4.w;
+          qq[r] = q4.x; qq[r + 1] = q4.y; qq[r + 2] = q4.z; qq[r + 3] = q4.w;
+        }
         const float xv = xcur[tt];
         float o;
         if (DELTA) {
-          const float* gg = &vecs[buf][tt][NV - 1][part * (R + 1)];
+          float gg[R];
+#pragma unroll
+          for (int r = 0; r < R; r += 4) {
+            const float4 g4 =
+                *reinterpret_cast<const float4*>(&vecs[buf][tt][NV - 1][part * RC_SHARE + r]);
+            gg[r] = g4.x; gg[r + 1] = g4.y; gg[r + 2] = g4.z; gg[r + 3] = g4.w;
+          }
           float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
 #pragma unroll
           for (int r = 0; r < R; r += 4) {
@@ -452,12 +469,16 @@ template <bool DELTA>
 static int launch_recurrence(const RecurrenceArgs& a, int n_seqs, int P, bool long_portions,
                              hipStream_t stream) {
   dim3 grid(n_seqs, a.H, (a.dv * P + 63) / 64), block(64);
+  // more waves than SIMDs (256 compute units of four): shorter chunks, more waves at once
+  const bool crowded = (long long)grid.x * grid.y * grid.z > 1024;
 #define ZA_RECURRENCE(PP)                                                                      \
   case PP:                                                                                     \
-    if (long_portions)                                                                         \
-      hipLaunchKernelGGL((matrix_recurrence_kernel<PP, DELTA, true>), grid, block, 0, stream, a);  \
+    if (long_portions && crowded)                                                              \
+      hipLaunchKernelGGL((matrix_recurrence_kernel<PP, DELTA, 1>), grid, block, 0, stream, a); \
+    else if (long_portions)                                                                    \
+      hipLaunchKernelGGL((matrix_recurrence_kernel<PP, DELTA, 2>), grid, block, 0, stream, a); \
     else                                                                                       \
-      hipLaunchKernelGGL((matrix_recurrence_kernel<PP, DELTA, false>), grid, block, 0, stream, a); \
+      hipLaunchKernelGGL((matrix_recurrence_kernel<PP, DELTA, 0>), grid, block, 0, stream, a); \
     break
   switch (P) {
     ZA_RECURRENCE(1);
