@@ -432,15 +432,16 @@ def test_small_kernels():
     from zig_ai_amd.kernels import ops
     dev = torch.device("cuda")
     gen = torch.Generator().manual_seed(0)
-    T, I = 9, 52
-    gu = (torch.randn(T, 2 * I, generator=gen) * 3).to(torch.bfloat16)
-    got = ops.clamped_glu(gu.to(dev), 2.0, 1.702, 1.0).cpu().double()
-    g = gu[:, :I].double().clamp(max=2.0)
-    u = gu[:, I:].double().clamp(-2.0, 2.0)
-    want = g * torch.sigmoid(1.702 * g) * (u + 1.0)
-    assert float((got - want).abs().max()) < 0.04
-    got = ops.clamped_glu(gu.float().to(dev), 2.0, 1.702, 1.0).cpu().double()
-    assert float((got - want).abs().max()) < 1e-5
+    T = 9
+    for I in (52, 56):          # element by element, and eight at a time
+        gu = (torch.randn(T, 2 * I, generator=gen) * 3).to(torch.bfloat16)
+        got = ops.clamped_glu(gu.to(dev), 2.0, 1.702, 1.0).cpu().double()
+        g = gu[:, :I].double().clamp(max=2.0)
+        u = gu[:, I:].double().clamp(-2.0, 2.0)
+        want = g * torch.sigmoid(1.702 * g) * (u + 1.0)
+        assert float((got - want).abs().max()) < 0.04
+        got = ops.clamped_glu(gu.float().to(dev), 2.0, 1.702, 1.0).cpu().double()
+        assert float((got - want).abs().max()) < 1e-5
     # gated group norm, both orders
     y = torch.randn(T, 96, generator=gen)
     gate = torch.randn(T, 96 + 8, generator=gen)

@@ -142,19 +142,47 @@ clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ out, int n_tokens, 
   out[idx] = from_f32<T>(g * (1.0f / (1.0f + expf(-alpha * g))) * (u + up_offset));
 }
 
+template <typename T>
+__global__ void __launch_bounds__(256)
+clamped_glu_vec8_kernel(const T* __restrict__ gu, T* __restrict__ out, int n_tokens, int inter,
+                        float limit, float alpha, float up_offset) {
+  const size_t idx = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  const size_t total = (size_t)n_tokens * inter;
+  if (idx >= total) return;
+  const size_t t = idx / inter, i = idx % inter;
+  float g[8], u[8], o[8];
+  load8<T>(gu + t * 2 * inter + i, g);
+  load8<T>(gu + t * 2 * inter + inter + i, u);
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    float gk = g[k], uk = u[k];
+    if (limit > 0.f) {
+      gk = fminf(gk, limit);
+      uk = fminf(fmaxf(uk, -limit), limit);
+    }
+    o[k] = gk * (1.0f / (1.0f + expf(-alpha * gk))) * (uk + up_offset);
+  }
+  store8<T>(out + idx, o);
+}
+
 extern "C" int za_clamped_glu(const void* gu, void* out, int dtype, int n_tokens, int inter,
                               float limit, float alpha, float up_offset, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   if (n_tokens < 0 || inter <= 0 || !gu || !out) return ZA_ERR_ARG;
   const size_t total = (size_t)n_tokens * inter;
-  dim3 grid((unsigned)((total + 255) / 256)), block(256);
-  if (dtype == 0)
-    hipLaunchKernelGGL((clamped_glu_kernel<float>), grid, block, 0, stream, (const float*)gu,
-                       (float*)out, n_tokens, inter, limit, alpha, up_offset);
-  else if (dtype == 1)
-    hipLaunchKernelGGL((clamped_glu_kernel<bf16_t>), grid, block, 0, stream, (const bf16_t*)gu,
-                       (bf16_t*)out, n_tokens, inter, limit, alpha, up_offset);
-  else
+  const bool vec = inter % 8 == 0;      // rows of both halves start on 16-byte boundaries
+  const size_t threads = vec ? total / 8 : total;
+  dim3 grid((unsigned)((threads + 255) / 256)), block(256);
+#define ZA_GLU(KERNEL, T)                                                                      \
+  hipLaunchKernelGGL((KERNEL<T>), grid, block, 0, stream, (const T*)gu, (T*)out, n_tokens, inter, \
+                     limit, alpha, up_offset)
+  if (dtype == 0) {
+    if (vec) ZA_GLU(clamped_glu_vec8_kernel, float); else ZA_GLU(clamped_glu_kernel, float);
+  } else if (dtype == 1) {
+    if (vec) ZA_GLU(clamped_glu_vec8_kernel, bf16_t); else ZA_GLU(clamped_glu_kernel, bf16_t);
+  } else {
     return ZA_ERR_UNSUPPORTED;
+  }
+#undef ZA_GLU
   return za_launch_status();
 }

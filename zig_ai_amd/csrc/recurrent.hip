@@ -62,15 +62,32 @@ causal_conv_silu_kernel(const T* __restrict__ x, int x_stride, int col0,
   const float b = bias ? bias[c] : 0.f;
   if ((int)blockIdx.y < body_blocks) {
     const int t0 = blockIdx.y * tokens_per_block;
+    // the L - 1 inputs before the token stay in registers from one token to the next
+    float before[RC_MAX_TAPS];
+    bool have = false;
     for (int t = t0; t < t0 + tokens_per_block && t < n_tokens; ++t) {
       const int rel = t - seq_start[token_seq[t]];
-      if (rel < L - 1) continue;
+      if (rel < L - 1) {
+        have = false;
+        continue;
+      }
+      if (!have) {
+#pragma unroll
+        for (int j = 0; j < RC_MAX_TAPS - 1; ++j)
+          before[j] = j < L - 1 ? to_f32<T>(x[(size_t)(t - (L - 1 - j)) * x_stride + col0 + c]) : 0.f;
+        have = true;
+      }
+      const float xi = to_f32<T>(x[(size_t)t * x_stride + col0 + c]);
       float acc = b;
 #pragma unroll
-      for (int j = 0; j < RC_MAX_TAPS; ++j)
-        if (j < L)
-          acc = fmaf(w[j], to_f32<T>(x[(size_t)(t - (L - 1 - j)) * x_stride + col0 + c]), acc);
+      for (int j = 0; j < RC_MAX_TAPS - 1; ++j)
+        if (j < L - 1) acc = fmaf(w[j], before[j], acc);
+      acc = fmaf(w[L - 1], xi, acc);
       out[(size_t)t * C + c] = silu_f(acc);
+#pragma unroll
+      for (int j = 0; j < RC_MAX_TAPS - 1; ++j)
+        if (j < L - 2) before[j] = before[j + 1];
+      if (L >= 2) before[L - 2] = xi;
     }
     return;
   }
@@ -115,7 +132,7 @@ extern "C" int za_causal_conv_silu(const void* x, int dtype, int x_stride, int c
       !slot_id || !out || col0 < 0 || col0 + C > x_stride || slot_stride < (long long)C * (L - 1))
     return ZA_ERR_ARG;
   if (L < 1 || L > RC_MAX_TAPS) return ZA_ERR_UNSUPPORTED;
-  const int tpb = 8;
+  const int tpb = 16;
   // (single tokens with a state to read: heads only)
   const int body = (n_tokens > n_seqs || L == 1) ? (n_tokens + tpb - 1) / tpb : 0;
   dim3 grid((C + 255) / 256, body + n_seqs), block(256);
