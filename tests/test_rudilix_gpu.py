@@ -173,6 +173,31 @@ def test_window_edges(window, rot):
             assert worst(got, want) < 2e-3, (name, page_size)
 
 
+# ------------------- key and value widths that the matrix-core attention kernels take
+@pytest.mark.parametrize("dim,window,rot", [(64, 40, 32), (128, 0, 128), (64, 130, 0)])
+def test_matrix_core_attention_with_gate(dim, window, rot):
+    att = ru.attention(heads=4, kv_heads=2, dim=dim, vdim=dim, window=window, rot_dims=rot,
+                       base=1000.0, scale=dim ** -0.5)
+    cfg = ru.config([ru.layer("parallel", ru.parallel(att, ru.delta(), 1.0, 0.5), ff=64)], width=128)
+    model, tensors = build(cfg, seed=6, dtype="bfloat16")
+    assert model.blocks[0].parts["left"].mfma
+    lengths = [200, 70, 3]
+    prompts = [ru.tokens(n, cfg["vocab"], 50 + i) for i, n in enumerate(lengths)]
+    want = plain_logits(cfg, tensors, prompts)
+    base = None
+    for name, schedule in (("whole", eu.whole(lengths)),
+                           ("bulk + tail", eu.bulk_then_single(lengths, tail=60)),
+                           ("portions", eu.changing_portions(lengths, seed=3)),
+                           ("mixed", eu.mixed(lengths, seed=1, max_live=3, decode_tail=30))):
+        runner = runner_for(model, page_size=16, tokens=512, slots=3)
+        got = eu.run_schedule(runner, prompts, schedule)
+        assert_bfloat16_close(torch.cat(got), torch.cat(want), name)
+        base = base or got
+        e = ru.row_error(torch.cat(got), torch.cat(base))
+        assert float(e.median()) < BF16_BETWEEN_MEDIAN and float(e.max()) < BF16_BETWEEN_WORST, \
+            (name, float(e.median()), float(e.max()))
+
+
 # ----------------------------------------------------------------- far tokens count
 @pytest.mark.parametrize("kind", ["mamba2", "channel_delta"])
 def test_far_tokens_reach_the_end(kind):

@@ -52,6 +52,8 @@ class LinearHead(Part):
         self.weight = tensors.get("weight")   # the model hands a tied head the embedding table
 
     def forward(self, x) -> torch.Tensor:
+        if not self.tied and self.weight.dtype == torch.bfloat16 and self.weight.shape[1] % 8:
+            self.weight = ops.projection_weight(self.weight)     # kept in 32-bit from now on
         ops.check_projection_weight(self.weight, "output head")
         return ops.linear(x, self.weight, out_dtype=torch.float32, tune=self.runtime.tune)
 

@@ -151,7 +151,6 @@ class GatedDeltaRule(Mixer):
         ops.recurrence_plan(d, dv)
         self.heads, self.kv_heads, self.head_dim, self.value_dim, self.taps = H, G, d, dv, L
         self.eps = float(params["norm_eps"])
-        self.out_scale = float(params.get("output_scale", 1.0))
         # one opening product: q | k | v | beta | decay_down | gate_down; each low-rank
         # block is filled up with zero rows to a multiple of 8, the input width that the
         # second product wants
