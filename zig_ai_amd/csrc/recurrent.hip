@@ -328,12 +328,16 @@ matrix_recurrence_kernel(RecurrenceArgs a) {
   const int lane_tt = lane / LPV, lane_i = (lane % LPV) * 4;
   float4 regs[NLOAD];
   float xnext[CH], snext = 0.f;
+  int chunk_left = 0;       // tokens of the portion from the requested chunk's start on
   auto request = [&](int c0) {
 #pragma unroll
     for (int j = 0; j < NLOAD; ++j) {
       const int v = j % NV, piece = (j / NV) % PIECES, group = j / (NV * PIECES);
       const int tt = group * TPL + lane_tt, i = piece * 256 + lane_i;
-      float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+      // (a chunk's places beyond the portion's end hold tokens that change nothing: no
+      // decay, nothing written, nothing read; the walk then needs no conditions)
+      const float idle = (DELTA && v == NV - 1 && c0 + tt >= n) ? 1.f : 0.f;
+      float4 x = make_float4(idle, idle, idle, idle);
       if (c0 + tt < n && i < dk) {
         const float* src = base[v] + (size_t)(start + c0 + tt) * stride + i;
         if (vec_loads) {
@@ -350,6 +354,8 @@ matrix_recurrence_kernel(RecurrenceArgs a) {
 #pragma unroll
     for (int tt = 0; tt < CH; ++tt)
       xnext[tt] = c0 + tt < n ? xsrc[(size_t)(start + c0 + tt) * a.conv_width] : 0.f;
+    snext = 0.f;
+    chunk_left = n - c0;
     if (lane < CH && c0 + lane < n) {
       const size_t t = start + c0 + lane;
       if (DELTA) {
@@ -373,8 +379,8 @@ matrix_recurrence_kernel(RecurrenceArgs a) {
         scal[buf][lane][0] = snext;
       } else {
         const float dt = softplus_f(snext + dtb);
-        scal[buf][lane][0] = expf(neg_A * dt);
-        scal[buf][lane][1] = dt;
+        scal[buf][lane][0] = lane < chunk_left ? expf(neg_A * dt) : 1.f;
+        scal[buf][lane][1] = lane < chunk_left ? dt : 0.f;
       }
     }
   };
@@ -393,8 +399,7 @@ matrix_recurrence_kernel(RecurrenceArgs a) {
                            // the walk wait for everything requested before it
 #pragma unroll
     for (int tt = 0; tt < CH; ++tt) {
-      result[tt] = 0.f;
-      if (tt < cn) {
+      {
         float kk[R], qq[R];
 #pragma unroll
         for (int r = 0; r < R; r += 4) {
