@@ -188,3 +188,45 @@ def row_error(got, want):
     d = d - d.mean(dim=1, keepdim=True)
     scale = (want - want.mean(dim=1, keepdim=True)).pow(2).mean().sqrt()
     return d.pow(2).mean(dim=1).sqrt() / scale
+
+
+def random_config(seed):
+    """A configuration drawn at random: layer order, every size and every constant."""
+    import random
+    rng = random.Random(seed)
+
+    def pick(*values):
+        return rng.choice(values)
+
+    def rand_delta():
+        kv = pick(1, 2, 3)
+        return delta(heads=kv * pick(1, 2), kv_heads=kv, dim=pick(8, 12, 16, 40, 72),
+                     vdim=pick(4, 8, 12, 24, 40), conv=pick(1, 2, 3, 4, 5))
+
+    def rand_attention():
+        kv = pick(1, 2, 3)
+        dim = pick(8, 16, 24, 40)
+        return attention(heads=kv * pick(1, 2, 4), kv_heads=kv, dim=dim, vdim=pick(8, 16, 32, 48),
+                         window=pick(0, 1, 2, 5, 17, 64, 500), rot_dims=pick(0, 2, dim // 2 // 2 * 2, dim),
+                         base=pick(10.0, 1000.0, 50000.0), scale=pick(0.1, 0.35, 0.7))
+
+    def rand_ssd():
+        groups = pick(1, 2, 3)
+        heads = groups * pick(1, 2)
+        vdim = pick(4, 8, 12, 24)
+        norm_groups = pick(*[g for g in (1, 2, 3, 4, heads) if (heads * vdim) % g == 0])
+        return ssd(heads=heads, vdim=vdim, state=pick(4, 8, 20, 48, 136), groups=groups,
+                   norm_groups=norm_groups, conv=pick(2, 3, 4, 6))
+
+    layers = []
+    for _ in range(pick(1, 2, 3, 4, 6)):
+        kind = pick("mamba2", "channel_delta", "parallel")
+        if kind == "mamba2":
+            mixer = rand_ssd()
+        elif kind == "channel_delta":
+            mixer = rand_delta()
+        else:
+            mixer = parallel(rand_attention(), rand_delta(), pick(0.3, 1.0, -0.8), pick(0.5, 1.0, 1.6))
+        layers.append(layer(kind, mixer, ff=pick(0, 8, 24, 100), limit=pick(0.3, 1.0, 4.0)))
+    return config(layers, width=pick(16, 24, 40, 64, 104), vocab=pick(11, 50, 203),
+                  residual_mult=pick(0.25, 1.0, 1.5), eps=pick(1e-6, 1e-5, 1e-3))

@@ -142,6 +142,36 @@ def test_schedules_bfloat16(which):
             (name, float(e.median()), float(e.max()))
 
 
+# ---------------------------------------- configurations drawn at random, both types
+@pytest.mark.parametrize("seed", range(12))
+def test_random_configurations(seed):
+    cfg = ru.random_config(seed)
+    lengths = [70, 1, 33, 12, 2]
+    prompts = [ru.tokens(n, cfg["vocab"], 90 + i) for i, n in enumerate(lengths)]
+    model, tensors = build(cfg, seed=seed)
+    want = plain_logits(cfg, tensors, prompts)
+    for name, schedule in (("whole", eu.whole(lengths)),
+                           ("portions", eu.changing_portions(lengths, seed=seed)),
+                           ("mixed", eu.mixed(lengths, seed=seed, max_live=3, decode_tail=9))):
+        peak = eu.peak_tokens(lengths, schedule, round_to=16)
+        runner = runner_for(model, page_size=4 if seed % 2 else 16, tokens=peak, slots=3)
+        got = eu.run_schedule(runner, prompts, schedule)
+        # (a model drawn with hardly any spread in its logits is measured against that
+        # spread all the same; the bound allows for it)
+        for i, (g, w) in enumerate(zip(got, want)):
+            assert worst(g, w) < 3 * F32_BOUND, (name, i, cfg)
+    # the same model in bfloat16 runs (odd widths fall back to 32-bit weights) and agrees
+    # with itself across schedules
+    model16, _ = build(cfg, seed=seed, dtype="bfloat16")
+    base = None
+    for schedule in (eu.whole(lengths), eu.mixed(lengths, seed=seed, max_live=3, decode_tail=9)):
+        got = eu.run_schedule(runner_for(model16, page_size=16, tokens=256, slots=3), prompts, schedule)
+        assert all(torch.isfinite(g).all() for g in got)
+        base = base or got
+        e = ru.row_error(torch.cat(got), torch.cat(base))
+        assert float(e.median()) < BF16_BETWEEN_MEDIAN, float(e.median())
+
+
 # --------------------------------------------- window edges, with scores that stand out
 def sharp_window_cfg(window, rot):
     # a scale that makes the softmax all but choose one key: a key wrongly seen or wrongly
