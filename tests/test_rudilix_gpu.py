@@ -228,6 +228,44 @@ def test_matrix_core_attention_with_gate(dim, window, rot):
             (name, float(e.median()), float(e.max()))
 
 
+# ---------------- a width at which a decode batch's opening products run the norm themselves
+def test_decode_batches_at_a_width_of_512():
+    from zig_ai_amd.kernels import ops
+    cfg = ru.config([ru.layer("parallel", ru.parallel()), ru.layer("mamba2", ru.ssd()),
+                     ru.layer("channel_delta", ru.delta(), ff=0)], width=512)
+    model, tensors = build(cfg, seed=13, dtype="bfloat16")
+    assert ops.normed_rows_fusable(3, 512)
+    lengths = [60, 25, 8]
+    prompts = [ru.tokens(n, cfg["vocab"], 70 + i) for i, n in enumerate(lengths)]
+    want = plain_logits(cfg, tensors, prompts)
+    whole = eu.run_schedule(runner_for(model, page_size=16, tokens=256), prompts, eu.whole(lengths))
+    # all three decode together from their fifth token on: steps of three rows
+    steps = [([(i, 0, 4) for i in range(3)], [])]
+    steps += [([(i, p, p + 1) for i, n in enumerate(lengths) if p < n],
+               [i for i, n in enumerate(lengths) if p == n - 1]) for p in range(4, max(lengths))]
+    got = eu.run_schedule(runner_for(model, page_size=16, tokens=256, graphs=False), prompts, steps)
+    # (such a step does take that form)
+    from zig_ai_amd.engine import StepEntry
+    runner = runner_for(model, page_size=16, tokens=64, graphs=False)
+    runner.admit("x")
+    runner.step([StepEntry("x", prompts[2][:4], [])])
+    ops.form_log = []
+    try:
+        runner.step([StepEntry("x", prompts[2][4:5], [0])])
+        assert any(r.get("norm_in_product") for r in ops.form_log if r["op"] == "linear")
+    finally:
+        ops.form_log = None
+    assert_bfloat16_close(torch.cat(got), torch.cat(want))
+    # (a product that runs the norm rounds x * weight and scales its sums, the norm as a
+    # kernel rounds x * scale * weight: the two runs differ as two roundings do, measured
+    # median 0.010, worst 0.038)
+    assert_bfloat16_close(torch.cat(got), torch.cat(whole))
+    # and replayed from graphs
+    again = eu.run_schedule(runner_for(model, page_size=16, tokens=256), prompts, steps)
+    e = ru.row_error(torch.cat(again), torch.cat(got))
+    assert float(e.max()) < BF16_BETWEEN_WORST
+
+
 # ----------------------------------------------------------------- far tokens count
 @pytest.mark.parametrize("kind", ["mamba2", "channel_delta"])
 def test_far_tokens_reach_the_end(kind):
