@@ -13,9 +13,10 @@ import json
 import os
 from typing import Any, Callable, Dict, Mapping
 
-from .spec import ConfigError, LayerCall, LayerSpec, ModelSpec, PartSpec  # noqa: F401
+from .spec import ConfigError, LayerCall, LayerSpec, ModelSpec, PartSpec, StreamStep  # noqa: F401
 from .lfm2 import Lfm2Config, feed_forward_width  # noqa: F401
 from .rudilix import RudilixConfig  # noqa: F401
+from .ranesun import RanesunConfig  # noqa: F401
 
 _ARCHITECTURES: Dict[str, Any] = {}
 
@@ -66,3 +67,4 @@ def load_config(model_dir: str):
 
 register_architecture("Lfm2ForCausalLM", Lfm2Config)
 register_architecture("Rudilix", RudilixConfig)
+register_architecture("Ranesun", RanesunConfig)

@@ -66,6 +66,16 @@ class LayerSpec:
 
 
 @dataclass(frozen=True)
+class StreamStep:
+    """Something that enters the residual stream right before a run-order entry:
+    ``part`` indexes ``ModelSpec.stream_parts``, ``args`` are the keywords its ``forward``
+    gets at this place (which row of its table, say)."""
+
+    part: int
+    args: Mapping[str, Any] = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
 class LayerCall:
     """One entry of the run order.
 
@@ -73,12 +83,14 @@ class LayerCall:
     call's mixer uses; two calls with the same ``cache`` share it, and only
     calls with ``writes_cache`` store into it (a reader of another layer's
     cache has ``writes_cache=False``).  ``cache=None`` gives the call an entry
-    of its own.
+    of its own (a layer that the run order names several times then has a cache,
+    or a state, per time it runs).  ``before``: see ``StreamStep``.
     """
 
     layer: int
     cache: Optional[int] = None
     writes_cache: bool = True
+    before: Optional[StreamStep] = None
 
 
 @dataclass(frozen=True)
@@ -93,6 +105,7 @@ class ModelSpec:
     lm_head: PartSpec
     max_position: int = 0
     ignored_tensors: Tuple[str, ...] = ()    # checkpoint names that may be there and are not read
+    stream_parts: Tuple[PartSpec, ...] = ()  # what run-order entries may name as ``before``
 
     def __post_init__(self) -> None:
         if not self.layers:
@@ -103,6 +116,9 @@ class ModelSpec:
             if not 0 <= call.layer < len(self.layers):
                 raise ConfigError(
                     f"run order names layer {call.layer}, but there are {len(self.layers)} layers")
+            if call.before is not None and not 0 <= call.before.part < len(self.stream_parts):
+                raise ConfigError(f"run order names stream part {call.before.part}, but there are "
+                                  f"{len(self.stream_parts)}")
 
     def resolved_schedule(self) -> Tuple[LayerCall, ...]:
         """The run order with every ``cache=None`` replaced by a fresh id."""
@@ -114,7 +130,7 @@ class ModelSpec:
                 while next_id in used:
                     next_id += 1
                 used.add(next_id)
-                out.append(LayerCall(call.layer, next_id, call.writes_cache))
+                out.append(LayerCall(call.layer, next_id, call.writes_cache, call.before))
             else:
                 out.append(call)
         return tuple(out)

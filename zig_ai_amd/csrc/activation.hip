@@ -186,3 +186,73 @@ extern "C" int za_clamped_glu(const void* gu, void* out, int dtype, int n_tokens
 #undef ZA_GLU
   return za_launch_status();
 }
+
+// A gated unit on the fused gate|up projection with a choice of activation:
+//   out[t, i] = act(gu[t, i]) * gu[t, I + i]
+//   act 0: silu(g) = g / (1 + exp(-g))
+//   act 1: gelu in its tanh form, 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))
+// in 32-bit.
+__device__ __forceinline__ float gate_act(float g, int act) {
+  if (act == 1) {
+    const float z = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+    return 0.5f * g * (1.0f + tanhf(z));
+  }
+  return g * (1.0f / (1.0f + expf(-g)));
+}
+
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+gated_unit_kernel(const T* __restrict__ gu, T* __restrict__ out, int n_tokens, int inter, int act) {
+  const size_t idx = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC;
+  const size_t total = (size_t)n_tokens * inter;
+  if (idx >= total) return;
+  const size_t t = idx / inter, i = idx % inter;
+  if (VEC == 8) {
+    float g[8], u[8], o[8];
+    load8<T>(gu + t * 2 * inter + i, g);
+    load8<T>(gu + t * 2 * inter + inter + i, u);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) o[k] = gate_act(g[k], act) * u[k];
+    store8<T>(out + idx, o);
+  } else {
+    const float g = to_f32<T>(gu[t * 2 * inter + i]);
+    const float u = to_f32<T>(gu[t * 2 * inter + inter + i]);
+    out[idx] = from_f32<T>(gate_act(g, act) * u);
+  }
+}
+
+extern "C" int za_gated_unit(const void* gu, void* out, int dtype, int n_tokens, int inter, int act,
+                             hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  if (n_tokens < 0 || inter <= 0 || !gu || !out || act < 0 || act > 1) return ZA_ERR_ARG;
+  const size_t total = (size_t)n_tokens * inter;
+  const bool vec = inter % 8 == 0;
+  const size_t threads = vec ? total / 8 : total;
+  dim3 grid((unsigned)((threads + 255) / 256)), block(256);
+#define ZA_UNIT(T, V)                                                                          \
+  hipLaunchKernelGGL((gated_unit_kernel<T, V>), grid, block, 0, stream, (const T*)gu, (T*)out, \
+                     n_tokens, inter, act)
+  if (dtype == 0) {
+    if (vec) ZA_UNIT(float, 8); else ZA_UNIT(float, 1);
+  } else if (dtype == 1) {
+    if (vec) ZA_UNIT(bf16_t, 8); else ZA_UNIT(bf16_t, 1);
+  } else {
+    return ZA_ERR_UNSUPPORTED;
+  }
+#undef ZA_UNIT
+  return za_launch_status();
+}
+
+// x <- x * s, 32-bit, in place (an output head's constant factor on its logits).
+__global__ void __launch_bounds__(256) scale_kernel(float* __restrict__ x, float s, size_t n) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx < n) x[idx] *= s;
+}
+
+extern "C" int za_scale(float* x, float s, long long n, hipStream_t stream) {
+  if (n == 0) return 0;
+  if (n < 0 || !x) return ZA_ERR_ARG;
+  hipLaunchKernelGGL(scale_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, s,
+                     (size_t)n);
+  return za_launch_status();
+}

@@ -29,6 +29,31 @@
 #include "common.h"
 #include "rope_math.h"
 
+// What a design may add to the score of a (query, key) pair and to the softmax; every
+// field's zero means "not there", and every kernel of this file takes the struct:
+//   temperature   q at position p counts (1 + qt_coef * ln(floor((p + 1) / qt_every) + 1))
+//                 times (qt_every > 0)
+//   cap           s <- softcap * tanh(s / softcap) after the scale (softcap > 0)
+//   sink          the softmax's denominator also holds exp(sink[head]): a term with no key
+//                 and no value, neither scaled nor capped, counted once however the
+//                 context is cut (the kernel that sees the whole context adds it at its end,
+//                 otherwise the merge of the ranges does)
+struct ScoreExtras {
+  float softcap;
+  const float* sink;
+  float qt_coef;
+  int qt_every;
+};
+
+__device__ __forceinline__ float query_temperature(const ScoreExtras& ex, int position) {
+  if (ex.qt_every <= 0) return 1.0f;
+  return 1.0f + ex.qt_coef * logf((float)((position + 1) / ex.qt_every) + 1.0f);
+}
+
+__device__ __forceinline__ float capped_score(const ScoreExtras& ex, float s) {
+  return ex.softcap > 0.f ? ex.softcap * tanhf(s / ex.softcap) : s;
+}
+
 #define AT_WAVES 4
 #define AT_RPW 8                     // rows per wave, at most
 #define AT_MAX_ROWS (AT_WAVES * AT_RPW)
@@ -44,7 +69,7 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
                        float* __restrict__ part_acc, float* __restrict__ part_ml, int nh, int nkv,
                        int d, int page_size, float scale, int window, int keys_per_split,
                        int nsplit, int dv, const T* __restrict__ gate, int gate_stride,
-                       int gate_col, float out_scale) {
+                       int gate_col, float out_scale, ScoreExtras ex) {
   // `dv`: width of a value (keys and queries have `d`); a page holds the keys of all
   // heads, [kv_head][offset][d], then the values turned round, [kv_head][dv][offset].
   // `gate`: when given, head h of token t is multiplied by
@@ -147,7 +172,7 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
           const float* kr = Ks + lane * ldk;
           float dot = 0.f;
           for (int dd = 0; dd < d; ++dd) dot = fmaf(qr[dd], kr[dd], dot);
-          if (valid) s = dot * scale;
+          if (valid) s = capped_score(ex, dot * query_temperature(ex, pos) * scale);
         }
         const float tmax = wave_max(s);
         const float m_new = fmaxf(m[lr], tmax);
@@ -183,6 +208,7 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
     if (r < rows) {
       const int tok = row0 + r / G, h = g * G + r % G;
       if (nsplit == 1) {
+        if (ex.sink) l[lr] += expf(ex.sink[h] - m[lr]);
         const float inv = l[lr] > 0.f ? 1.0f / l[lr] : 0.f;
         float mult = 1.0f;
         if (gate) {
@@ -217,7 +243,9 @@ paged_attention_kernel(const T* __restrict__ q, T* __restrict__ out, const T* __
 template <typename T>
 __global__ void __launch_bounds__(64)
 attention_combine_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-                         T* __restrict__ out, int d, int nsplit, int base2) {
+                         T* __restrict__ out, int d, int nsplit, int base2,
+                         const float* __restrict__ sink, int nh) {
+  // `sink`: one number a head whose exponential joins the denominator once (none if null)
   const size_t row = blockIdx.x;  // token * nh + head
   const int lane = threadIdx.x;
   float mx = -INFINITY;
@@ -238,6 +266,10 @@ attention_combine_kernel(const float* __restrict__ part_acc, const float* __rest
       const int dd = lane + 64 * c;
       if (dd < d) acc[c] = fmaf(pa[dd], w, acc[c]);
     }
+  }
+  if (sink && mx > -INFINITY) {
+    const float sk = sink[row % nh];
+    total += base2 ? exp2f(sk * 1.4426950408889634f - mx) : expf(sk - mx);
   }
   const float inv = total > 0.f ? 1.0f / total : 0.f;
 #pragma unroll
@@ -1062,7 +1094,8 @@ static int launch_attention(const void* q, void* out, const void* kv, const int*
                             const int* wi_row0, const int* wi_count, int n_items, float* part_acc,
                             float* part_ml, int nh, int nkv, int d, int page_size, float scale,
                             int window, int keys_per_split, int nsplit, int dv, const void* gate,
-                            int gate_stride, int gate_col, float out_scale, hipStream_t stream) {
+                            int gate_stride, int gate_col, float out_scale, ScoreExtras ex,
+                            hipStream_t stream) {
   const size_t shmem = ((size_t)KT * (d + 1) + (size_t)KT * (dv + 1) + (size_t)AT_MAX_ROWS * d +
                         AT_WAVES * 64) * sizeof(float);
   auto kernel = paged_attention_kernel<T, KT>;
@@ -1077,7 +1110,7 @@ static int launch_attention(const void* q, void* out, const void* kv, const int*
   hipLaunchKernelGGL(kernel, grid, block, shmem, stream, (const T*)q, (T*)out, (const T*)kv,
                      block_table, bt_stride, positions, wi_seq, wi_row0, wi_count, part_acc,
                      part_ml, nh, nkv, d, page_size, scale, window, keys_per_split, nsplit, dv,
-                     (const T*)gate, gate_stride, gate_col, out_scale);
+                     (const T*)gate, gate_stride, gate_col, out_scale, ex);
   return za_launch_status();
 }
 
@@ -1121,7 +1154,7 @@ static int paged_attention_any(const void* q, void* out, const void* kv, const i
                                int n_tokens, float* part_acc, float* part_ml, int dtype, int nh,
                                int nkv, int d, int page_size, float scale, int window,
                                int keys_per_split, int nsplit, int dv, const void* gate,
-                               int gate_stride, int gate_col, float out_scale,
+                               int gate_stride, int gate_col, float out_scale, ScoreExtras ex,
                                hipStream_t stream);
 
 // dtype codes: 0 = float32, 1 = bfloat16
@@ -1134,7 +1167,7 @@ extern "C" int za_paged_attention(const void* q, void* out, const void* kv, cons
   return paged_attention_any(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0,
                              wi_count, n_items, n_tokens, part_acc, part_ml, dtype, nh, nkv, d,
                              page_size, scale, window, keys_per_split, nsplit, d, nullptr, 0, 0,
-                             1.0f, stream);
+                             1.0f, ScoreExtras{0.f, nullptr, 0.f, 0}, stream);
 }
 
 // The same with values of width `dv` (a page: keys [kv_head][offset][d], then values
@@ -1153,7 +1186,27 @@ extern "C" int za_paged_attention_gated(const void* q, void* out, const void* kv
   return paged_attention_any(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0,
                              wi_count, n_items, n_tokens, part_acc, part_ml, dtype, nh, nkv, d,
                              page_size, scale, window, keys_per_split, nsplit, dv, gate,
-                             gate_stride, gate_col, out_scale, stream);
+                             gate_stride, gate_col, out_scale, ScoreExtras{0.f, nullptr, 0.f, 0},
+                             stream);
+}
+
+// The same with what `ScoreExtras` describes: a cap on the scores, a sink a head
+// (`sink`: nh 32-bit numbers, or null) and a temperature on the queries by position.
+extern "C" int za_paged_attention_shaped(const void* q, void* out, const void* kv,
+                                         const int* block_table, int bt_stride,
+                                         const int* positions, const int* wi_seq,
+                                         const int* wi_row0, const int* wi_count, int n_items,
+                                         int n_tokens, float* part_acc, float* part_ml, int dtype,
+                                         int nh, int nkv, int d, int dv, int page_size, float scale,
+                                         int window, int keys_per_split, int nsplit,
+                                         float softcap, const float* sink, float qt_coef,
+                                         int qt_every, hipStream_t stream) {
+  if (dv <= 0 || dv % 8 != 0 || dv > AT_MAX_D || softcap < 0.f || qt_every < 0)
+    return ZA_ERR_UNSUPPORTED;
+  return paged_attention_any(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0,
+                             wi_count, n_items, n_tokens, part_acc, part_ml, dtype, nh, nkv, d,
+                             page_size, scale, window, keys_per_split, nsplit, dv, nullptr, 0, 0,
+                             1.0f, ScoreExtras{softcap, sink, qt_coef, qt_every}, stream);
 }
 
 static int paged_attention_any(const void* q, void* out, const void* kv, const int* block_table,
@@ -1162,7 +1215,7 @@ static int paged_attention_any(const void* q, void* out, const void* kv, const i
                                int n_tokens, float* part_acc, float* part_ml, int dtype, int nh,
                                int nkv, int d, int page_size, float scale, int window,
                                int keys_per_split, int nsplit, int dv, const void* gate,
-                               int gate_stride, int gate_col, float out_scale,
+                               int gate_stride, int gate_col, float out_scale, ScoreExtras ex,
                                hipStream_t stream) {
   if (n_items == 0 || n_tokens == 0) return 0;
   if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || d <= 0 || page_size <= 0 ||
@@ -1177,7 +1230,7 @@ static int paged_attention_any(const void* q, void* out, const void* kv, const i
 #define ZA_AT_ARGS                                                                            \
   q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0, wi_count, n_items, part_acc, \
       part_ml, nh, nkv, d, page_size, scale, window, keys_per_split, nsplit, dv, gate,         \
-      gate_stride, gate_col, out_scale, stream
+      gate_stride, gate_col, out_scale, ex, stream
   const bool small = d <= 128 && dv <= 128;
   if (dtype == 0) {
     rc = small ? launch_attention<float, 64>(ZA_AT_ARGS) : launch_attention<float, 32>(ZA_AT_ARGS);
@@ -1192,10 +1245,10 @@ static int paged_attention_any(const void* q, void* out, const void* kv, const i
   dim3 grid((unsigned)((size_t)n_tokens * nh)), block(64);
   if (dtype == 0)
     hipLaunchKernelGGL((attention_combine_kernel<float>), grid, block, 0, stream, part_acc,
-                       part_ml, (float*)out, dv, nsplit, 0);
+                       part_ml, (float*)out, dv, nsplit, 0, ex.sink, nh);
   else
     hipLaunchKernelGGL((attention_combine_kernel<bf16_t>), grid, block, 0, stream, part_acc,
-                       part_ml, (bf16_t*)out, dv, nsplit, 0);
+                       part_ml, (bf16_t*)out, dv, nsplit, 0, ex.sink, nh);
   rc = za_launch_status();
   if (rc != 0 || !gate) return rc;
   return za_head_gate(out, gate, dtype, gate_stride, gate_col, n_tokens, nh, dv, out_scale, stream);
@@ -1230,7 +1283,7 @@ static int launch_attention_mfma(const void* q, void* out, const void* kv, const
   if (rc != 0 || nsplit == 1) return rc;
   dim3 cgrid((unsigned)((size_t)n_tokens * nh)), cblock(64);
   hipLaunchKernelGGL((attention_combine_kernel<bf16_t>), cgrid, cblock, 0, stream, part_acc,
-                     part_ml, (bf16_t*)out, D, nsplit, 1);
+                     part_ml, (bf16_t*)out, D, nsplit, 1, nullptr, 1);
   return za_launch_status();
 }
 
@@ -1303,7 +1356,7 @@ static int launch_decode_mfma(const void* q, void* out, const void* kv, const in
   if (rc != 0 || nsplit == 1 || !combine) return rc;
   dim3 cgrid((unsigned)((size_t)n_tokens * nh)), cblock(64);
   hipLaunchKernelGGL((attention_combine_kernel<bf16_t>), cgrid, cblock, 0, stream, part_acc,
-                     part_ml, (bf16_t*)out, d, nsplit, 1);
+                     part_ml, (bf16_t*)out, d, nsplit, 1, nullptr, 1);
   return za_launch_status();
 }
 
@@ -1315,7 +1368,7 @@ extern "C" int za_attention_combine(const float* part_acc, const float* part_ml,
   if (rows < 0 || d <= 0 || d > AT_MAX_D || nsplit < 1 || !part_acc || !part_ml || !out)
     return ZA_ERR_ARG;
   hipLaunchKernelGGL((attention_combine_kernel<bf16_t>), dim3((unsigned)rows), dim3(64), 0, stream,
-                     part_acc, part_ml, (bf16_t*)out, d, nsplit, 1);
+                     part_acc, part_ml, (bf16_t*)out, d, nsplit, 1, nullptr, 1);
   return za_launch_status();
 }
 

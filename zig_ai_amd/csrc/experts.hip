@@ -1,0 +1,288 @@
+// A feed-forward of many small experts of which each token uses a few: the lists of
+// who goes where, and products of every expert's rows with that expert's weights in one
+// launch ("grouped" products).
+//
+// A step has A = T * top assignments; assignment a = t * top + j is token t's j-th expert.
+//
+// 1. expert_lists: one workgroup an expert walks the assignments in order and writes the
+//    ones that name it, ascending, into lists[e][0 .. counts[e]).  No atomics, nothing to
+//    clear beforehand, and the lists do not depend on the order in which anything ran.
+//    Where an expert comes from is the caller's business: here a table indexed by the
+//    token id, [vocab][top] (a router's top-k output [T][top] takes the same kernel with
+//    the row index in place of the token id).
+//
+// 2. grouped_gemm: for every expert e and every tile of TM of its assignments,
+//        out[dst(a)] = f(src[a / src_div] @ W[e]^T) * out_scale
+//    src_div = top reads the tokens' rows, src_div = 1 rows that are already one an
+//    assignment.  dst(a) = a, or, `stacked`, (a % top) * T + a / top: a stack [top][T][N]
+//    of 32-bit partial results, which the norm that follows adds up in its order (so the
+//    weighted sum over a token's experts is taken in 32-bit and costs no kernel).
+//    f: nothing, or the square of relu.
+//    How many tiles there are is known on the device only; the grid is the upper bound
+//    ceil(A / TM) + E and a workgroup beyond the last tile leaves at once.
+//    Every output element is a sum over k in an order fixed by K alone: a token's result
+//    does not depend on which other tokens share its expert or its tile.
+//      bfloat16: matrix cores (v_mfma_f32_16x16x32_bf16), operands straight from memory
+//      into the fragments; TM = 64 (four waves, 16 rows x 64 columns each) for steps with
+//      prompt portions, TM = 16 (four waves, 16 columns each) for decode batches, where an
+//      expert has a token or two and the weights are all that moves.
+//      32-bit: LDS-tiled FMA, 64 x 64 tiles (no matrix-core rounding mode).
+#include "common.h"
+
+#define EX_MAX_EXPERTS 1024
+
+// lists: int [E][A]; counts: int [E].  `ids` names the table's row for each token (null:
+// the token's own index); an id outside [0, rows) names no expert.
+__global__ void __launch_bounds__(256)
+expert_lists_kernel(const int* __restrict__ ids, const int* __restrict__ table, int rows, int T,
+                    int top, int* __restrict__ lists, int* __restrict__ counts) {
+  __shared__ int wave_total[4];
+  const int e = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int A = T * top;
+  int* mine = lists + (size_t)e * A;
+  int running = 0;
+  for (int base = 0; base < A; base += 256) {
+    const int a = base + tid;
+    bool hit = false;
+    if (a < A) {
+      const int t = a / top, id = ids ? ids[t] : t;
+      hit = id >= 0 && id < rows && table[(size_t)id * top + a % top] == e;
+    }
+    const unsigned long long mask = __ballot(hit);
+    const int before = __popcll(mask & ((1ull << lane) - 1ull));
+    __syncthreads();      // the last round's totals have been read
+    if (lane == 0) wave_total[wave] = __popcll(mask);
+    __syncthreads();
+    int offset = running;
+    for (int w = 0; w < wave; ++w) offset += wave_total[w];
+    if (hit) mine[offset + before] = a;
+    running += wave_total[0] + wave_total[1] + wave_total[2] + wave_total[3];
+  }
+  if (tid == 0) counts[e] = running;
+}
+
+extern "C" int za_expert_lists(const int* ids, const int* table, int rows, int n_tokens, int top,
+                               int experts, int* lists, int* counts, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  if (n_tokens < 0 || top <= 0 || experts <= 0 || rows <= 0 || !table || !lists || !counts)
+    return ZA_ERR_ARG;
+  if (experts > EX_MAX_EXPERTS) return ZA_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(expert_lists_kernel, dim3(experts), dim3(256), 0, stream, ids, table, rows,
+                     n_tokens, top, lists, counts);
+  return za_launch_status();
+}
+
+struct GroupedArgs {
+  const void* src;       // [rows][K]
+  const void* W;         // [E][N][K]
+  const int* lists;      // [E][A]
+  const int* counts;     // [E]
+  void* out;
+  int A, T, top, E, N, K;
+  int src_div, stacked, act;
+  float out_scale;
+};
+
+// The expert and the tile within it that workgroup `b` serves; false when there is none.
+template <int TM>
+__device__ __forceinline__ bool find_tile(const int* __restrict__ counts, int E, int b, int* e_out,
+                                          int* tile_out, int* count_out) {
+  int first = 0;
+  for (int e = 0; e < E; ++e) {
+    const int c = counts[e], tiles = (c + TM - 1) / TM;
+    if (b < first + tiles) {
+      *e_out = e;
+      *tile_out = b - first;
+      *count_out = c;
+      return true;
+    }
+    first += tiles;
+  }
+  return false;
+}
+
+__device__ __forceinline__ float expert_act(float v, int act) {
+  if (act == 1) {
+    const float r = fmaxf(v, 0.f);
+    return r * r;
+  }
+  return v;
+}
+
+__device__ __forceinline__ size_t dst_row(const GroupedArgs& g, int a) {
+  return g.stacked ? (size_t)(a % g.top) * g.T + a / g.top : (size_t)a;
+}
+
+// Operand layout of v_mfma_f32_16x16x32_bf16: lane l supplies row (l % 16), k-slots
+// (l / 16) * 8 .. + 7 of either operand and receives rows (l / 16) * 4 .. + 3, column
+// (l % 16) of the product.
+template <int TM, typename TO>
+__global__ void __launch_bounds__(256)
+grouped_gemm_bf16_kernel(GroupedArgs g) {
+  constexpr int WM = TM / 16;          // waves along the rows
+  constexpr int WN = 4 / WM;           // waves along the columns
+  constexpr int NT = 4 / WN;           // 16-column tiles a wave
+  int e, tile, count;
+  if (!find_tile<TM>(g.counts, g.E, blockIdx.x, &e, &tile, &count)) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave % WM, wn = wave / WM;
+  const int r16 = lane & 15, kq = lane >> 4;
+  const int n0 = blockIdx.y * 64 + wn * NT * 16;
+  const int* mine = g.lists + (size_t)e * g.A;
+  const int K = g.K, N = g.N;
+
+  const int row = tile * TM + wm * 16 + r16;
+  const bool row_ok = row < count;
+  const bf16_t* arow = (const bf16_t*)g.src + (size_t)(row_ok ? mine[row] / g.src_div : 0) * K;
+  const bf16_t* wbase = (const bf16_t*)g.W + (size_t)e * N * K;
+  const bf16_t* wrow[NT];
+  bool col_ok[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int n = n0 + j * 16 + r16;
+    col_ok[j] = n < N;
+    wrow[j] = wbase + (size_t)(col_ok[j] ? n : 0) * K;
+  }
+  f32x4_t acc[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) acc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  for (int k0 = 0; k0 < K; k0 += 64) {
+    // two steps of 32 a round: their loads are all requested before the first product
+    bf16x8_t fa[2], fw[2][NT];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int k = k0 + s * 32 + kq * 8;
+      const bool k_ok = k < K;           // K is a multiple of 8: a piece is inside or outside
+      fa[s] = (row_ok && k_ok) ? *reinterpret_cast<const bf16x8_t*>(arow + k) : zero;
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        fw[s][j] = (col_ok[j] && k_ok) ? *reinterpret_cast<const bf16x8_t*>(wrow[j] + k) : zero;
+    }
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[s], fw[s][j], acc[j], 0, 0, 0);
+  }
+
+  TO* out = (TO*)g.out;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = tile * TM + wm * 16 + kq * 4 + i;
+    if (r >= count) continue;
+    const size_t d = dst_row(g, mine[r]);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const int n = n0 + j * 16 + r16;
+      if (n < N) out[d * N + n] = from_f32<TO>(expert_act(acc[j][i], g.act) * g.out_scale);
+    }
+  }
+}
+
+// 32-bit weights (src of either type): 64 x 64 tiles through LDS, plain FMA.
+template <typename TA, typename TO>
+__global__ void __launch_bounds__(256)
+grouped_gemm_f32_kernel(GroupedArgs g) {
+  __shared__ float As[16][64 + 4];
+  __shared__ float Ws[16][64 + 4];
+  int e, tile, count;
+  if (!find_tile<64>(g.counts, g.E, blockIdx.x, &e, &tile, &count)) return;
+  const int tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
+  const int n0 = blockIdx.y * 64;
+  const int* mine = g.lists + (size_t)e * g.A;
+  const int K = g.K, N = g.N;
+  const float* W = (const float*)g.W + (size_t)e * N * K;
+  const int lrow = tid / 4, lk = (tid % 4) * 4;
+  const int arow_idx = tile * 64 + lrow;
+  const bool a_ok = arow_idx < count;
+  const TA* arow = (const TA*)g.src + (size_t)(a_ok ? mine[arow_idx] / g.src_div : 0) * K;
+  const bool w_ok = n0 + lrow < N;
+  const float* wrow = W + (size_t)(w_ok ? n0 + lrow : 0) * K;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+  for (int k0 = 0; k0 < K; k0 += 16) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = k0 + lk + j;
+      As[lk + j][lrow] = (a_ok && k < K) ? to_f32<TA>(arow[k]) : 0.f;
+      Ws[lk + j][lrow] = (w_ok && k < K) ? wrow[k] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 16; ++kk) {
+      float a[4], w[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = Ws[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+  TO* out = (TO*)g.out;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = tile * 64 + ty * 4 + i;
+    if (r >= count) continue;
+    const size_t d = dst_row(g, mine[r]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n < N) out[d * N + n] = from_f32<TO>(expert_act(acc[i][j], g.act) * g.out_scale);
+    }
+  }
+}
+
+// dtype codes: 0 = float32, 1 = bfloat16.  `src` has `src_rows` rows of K elements; the
+// lists name assignments below n_tokens * top, so src_rows >= n_tokens (src_div == top) or
+// >= n_tokens * top (src_div == 1).
+extern "C" int za_grouped_gemm(const void* src, int src_dtype, long long src_rows, const void* W,
+                               int w_dtype, const int* lists, const int* counts, void* out,
+                               int out_dtype, int n_tokens, int top, int experts, int N, int K,
+                               int src_div, int stacked, int act, float out_scale,
+                               hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  if (n_tokens < 0 || top <= 0 || experts <= 0 || N <= 0 || K <= 0 || !src || !W || !lists ||
+      !counts || !out || (src_div != 1 && src_div != top) || act < 0 || act > 1)
+    return ZA_ERR_ARG;
+  const long long A = (long long)n_tokens * top;
+  if (src_rows < (src_div == 1 ? A : (long long)n_tokens) || A > 0x7fffffff) return ZA_ERR_ARG;
+  if (experts > EX_MAX_EXPERTS) return ZA_ERR_UNSUPPORTED;
+  if (stacked && out_dtype != 0) return ZA_ERR_UNSUPPORTED;
+  GroupedArgs g{src, W, lists, counts, out, (int)A, n_tokens, top, experts, N, K,
+                src_div, stacked, act, out_scale};
+  const unsigned ntiles = (unsigned)((N + 63) / 64);
+  if (w_dtype == 1) {
+    if (src_dtype != 1 || K % 8 != 0) return ZA_ERR_UNSUPPORTED;
+    // a decode batch (an expert has a token or two): tiles of 16 rows
+    const bool small = A <= 4LL * experts || A <= 64;
+    const int TM = small ? 16 : 64;
+    dim3 grid((unsigned)((A + TM - 1) / TM + experts), ntiles), block(256);
+#define ZA_GG(TMM, TO) \
+  hipLaunchKernelGGL((grouped_gemm_bf16_kernel<TMM, TO>), grid, block, 0, stream, g)
+    if (out_dtype == 0) { if (small) ZA_GG(16, float); else ZA_GG(64, float); }
+    else if (out_dtype == 1) { if (small) ZA_GG(16, bf16_t); else ZA_GG(64, bf16_t); }
+    else return ZA_ERR_UNSUPPORTED;
+#undef ZA_GG
+    return za_launch_status();
+  }
+  if (w_dtype != 0) return ZA_ERR_UNSUPPORTED;
+  dim3 grid((unsigned)((A + 63) / 64 + experts), ntiles), block(256);
+#define ZA_GF(TA, TO) \
+  hipLaunchKernelGGL((grouped_gemm_f32_kernel<TA, TO>), grid, block, 0, stream, g)
+  if (src_dtype == 0 && out_dtype == 0) ZA_GF(float, float);
+  else if (src_dtype == 1 && out_dtype == 0) ZA_GF(bf16_t, float);
+  else if (src_dtype == 1 && out_dtype == 1) ZA_GF(bf16_t, bf16_t);
+  else if (src_dtype == 0 && out_dtype == 1) ZA_GF(float, bf16_t);
+  else return ZA_ERR_UNSUPPORTED;
+#undef ZA_GF
+  return za_launch_status();
+}

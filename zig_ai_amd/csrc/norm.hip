@@ -76,7 +76,8 @@ __global__ void __launch_bounds__(256)
 add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
                    const float* __restrict__ weight, TO* __restrict__ out,
                    const int* __restrict__ rows, int width, float eps, int write_residual,
-                   int n_partials, size_t partial_stride) {
+                   int n_partials, size_t partial_stride, const float* __restrict__ bias,
+                   int center) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
@@ -84,12 +85,29 @@ add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
   const TD* dl = delta ? delta + src * width : nullptr;
   TO* o = out + (size_t)r * width;
 
-  float ss = 0.f;
+  float ss = 0.f, sum = 0.f;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float h = x ? x[i] : 0.f;
     if (dl) h += delta_at<TD>(dl, i, n_partials, partial_stride);
     if (write_residual) x[i] = h;
     ss += h * h;
+    sum += h;
+  }
+  float mean = 0.f;
+  if (center) {
+    // a layer norm: the squared deviations from the mean, summed in a pass of their own
+    mean = block_sum(sum, scratch) / (float)width;
+    ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+      float h;
+      if (write_residual) {
+        h = x[i];
+      } else {
+        h = x ? x[i] : 0.f;
+        if (dl) h += delta_at<TD>(dl, i, n_partials, partial_stride);
+      }
+      ss += (h - mean) * (h - mean);
+    }
   }
   ss = block_sum(ss, scratch);
   const float scale = 1.0f / sqrtf(ss / (float)width + eps);
@@ -101,7 +119,8 @@ add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
       h = x ? x[i] : 0.f;
       if (dl) h += delta_at<TD>(dl, i, n_partials, partial_stride);
     }
-    o[i] = from_f32<TO>(h * scale * weight[i]);
+    const float y = (h - mean) * scale * weight[i];
+    o[i] = from_f32<TO>(bias ? y + bias[i] : y);
   }
 }
 
@@ -112,7 +131,8 @@ __global__ void __launch_bounds__(256)
 add_rmsnorm_regs_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
                         const float* __restrict__ weight, TO* __restrict__ out,
                         const int* __restrict__ rows, int width, float eps, int write_residual,
-                        int n_partials, size_t partial_stride) {
+                        int n_partials, size_t partial_stride, const float* __restrict__ bias,
+                        int center) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
@@ -120,7 +140,7 @@ add_rmsnorm_regs_kernel(float* __restrict__ residual, const TD* __restrict__ del
   const TD* dl = delta ? delta + src * width : nullptr;
   TO* o = out + (size_t)r * width;
   float h[VPT][4];
-  float ss = 0.f;
+  float ss = 0.f, sum = 0.f;
 #pragma unroll
   for (int v = 0; v < VPT; ++v) {
     const int i = (threadIdx.x + v * 256) * 4;
@@ -140,7 +160,26 @@ add_rmsnorm_regs_kernel(float* __restrict__ residual, const TD* __restrict__ del
       if (write_residual)
         *reinterpret_cast<float4*>(x + i) = make_float4(h[v][0], h[v][1], h[v][2], h[v][3]);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) ss += h[v][e] * h[v][e];
+      for (int e = 0; e < 4; ++e) {
+        ss += h[v][e] * h[v][e];
+        sum += h[v][e];
+      }
+    }
+  }
+  if (center) {
+    // a layer norm: the row (already stored, if it is to be) becomes its deviations
+    const float mean = block_sum(sum, scratch) / (float)width;
+    ss = 0.f;
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) {
+      const int i = (threadIdx.x + v * 256) * 4;
+      if (i < width) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          h[v][e] -= mean;
+          ss += h[v][e] * h[v][e];
+        }
+      }
     }
   }
   ss = block_sum(ss, scratch);
@@ -150,8 +189,12 @@ add_rmsnorm_regs_kernel(float* __restrict__ residual, const TD* __restrict__ del
     const int i = (threadIdx.x + v * 256) * 4;
     if (i < width) {
       const float4 w = *reinterpret_cast<const float4*>(weight + i);
-      const float y[4] = {h[v][0] * scale * w.x, h[v][1] * scale * w.y, h[v][2] * scale * w.z,
-                          h[v][3] * scale * w.w};
+      float y[4] = {h[v][0] * scale * w.x, h[v][1] * scale * w.y, h[v][2] * scale * w.z,
+                    h[v][3] * scale * w.w};
+      if (bias) {
+        const float4 b = *reinterpret_cast<const float4*>(bias + i);
+        y[0] += b.x; y[1] += b.y; y[2] += b.z; y[3] += b.w;
+      }
       store4<TO>(o + i, y);
     }
   }
@@ -174,10 +217,10 @@ embed_gather_kernel(const int* __restrict__ tokens, const T* __restrict__ table,
 }
 
 // dtype codes: 0 = float32, 1 = bfloat16
-extern "C" int za_add_rmsnorm(void* residual, const void* delta, int delta_dtype,
-                              const float* weight, void* out, int out_dtype, const int* rows,
-                              int n_rows, int width, float eps, int write_residual,
-                              int n_partials, long long partial_stride, hipStream_t stream) {
+static int add_norm_any(void* residual, const void* delta, int delta_dtype, const float* weight,
+                        const float* bias, int center, void* out, int out_dtype, const int* rows,
+                        int n_rows, int width, float eps, int write_residual, int n_partials,
+                        long long partial_stride, hipStream_t stream) {
   if (n_rows == 0) return 0;
   if (n_rows < 0 || width <= 0 || (!residual && !delta) || !weight || !out || n_partials < 1)
     return ZA_ERR_ARG;
@@ -189,7 +232,7 @@ extern "C" int za_add_rmsnorm(void* residual, const void* delta, int delta_dtype
 #define ZA_NORM_LAUNCH(KERNEL, TD, TO)                                                      \
   hipLaunchKernelGGL((KERNEL), grid, block, 0, stream, res, (const TD*)delta, weight,       \
                      (TO*)out, rows, width, eps, write_residual, n_partials,                \
-                     (size_t)partial_stride)
+                     (size_t)partial_stride, bias, center)
 #define ZA_NORM_CASE(DD, TD, OD, TO)                                                        \
   if (delta_dtype == DD && out_dtype == OD) {                                               \
     if (vpt == 1) ZA_NORM_LAUNCH((add_rmsnorm_regs_kernel<TD, TO, 1>), TD, TO);             \
@@ -205,6 +248,62 @@ extern "C" int za_add_rmsnorm(void* residual, const void* delta, int delta_dtype
 #undef ZA_NORM_CASE
 #undef ZA_NORM_LAUNCH
   return ZA_ERR_UNSUPPORTED;
+}
+
+extern "C" int za_add_rmsnorm(void* residual, const void* delta, int delta_dtype,
+                              const float* weight, void* out, int out_dtype, const int* rows,
+                              int n_rows, int width, float eps, int write_residual,
+                              int n_partials, long long partial_stride, hipStream_t stream) {
+  return add_norm_any(residual, delta, delta_dtype, weight, nullptr, 0, out, out_dtype, rows,
+                      n_rows, width, eps, write_residual, n_partials, partial_stride, stream);
+}
+
+// The same with the mean taken off first and a bias added last (a layer norm):
+//   out = (h - mean(h)) / sqrt(mean((h - mean(h))^2) + eps) * weight + bias
+extern "C" int za_add_layernorm(void* residual, const void* delta, int delta_dtype,
+                                const float* weight, const float* bias, void* out, int out_dtype,
+                                const int* rows, int n_rows, int width, float eps,
+                                int write_residual, int n_partials, long long partial_stride,
+                                hipStream_t stream) {
+  return add_norm_any(residual, delta, delta_dtype, weight, bias, 1, out, out_dtype, rows,
+                      n_rows, width, eps, write_residual, n_partials, partial_stride, stream);
+}
+
+// x[t] <- x[t] + delta[t] (a tensor or a stack of partial sums, may be absent) + origin[t]
+// (32-bit, may be absent) + vec (32-bit [width], may be absent): what enters the stream
+// between two run-order entries.
+template <typename TD>
+__global__ void __launch_bounds__(256)
+stream_add_kernel(float* __restrict__ x, const TD* __restrict__ delta, int n_partials,
+                  size_t partial_stride, const float* __restrict__ origin,
+                  const float* __restrict__ vec, int width, size_t total) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  float h = x[i];
+  if (delta) h += delta_at<TD>(delta, i, n_partials, partial_stride);
+  if (origin) h += origin[i];
+  if (vec) h += vec[i % width];
+  x[i] = h;
+}
+
+extern "C" int za_stream_add(float* x, const void* delta, int delta_dtype, int n_partials,
+                             long long partial_stride, const float* origin, const float* vec,
+                             int n_rows, int width, hipStream_t stream) {
+  if (n_rows == 0) return 0;
+  if (n_rows < 0 || width <= 0 || !x || n_partials < 1) return ZA_ERR_ARG;
+  if (n_partials > 1 && (!delta || partial_stride <= 0)) return ZA_ERR_ARG;
+  const size_t total = (size_t)n_rows * width;
+  dim3 grid((unsigned)((total + 255) / 256)), block(256);
+  if (delta_dtype == 0)
+    hipLaunchKernelGGL((stream_add_kernel<float>), grid, block, 0, stream, x, (const float*)delta,
+                       n_partials, (size_t)partial_stride, origin, vec, width, total);
+  else if (delta_dtype == 1)
+    hipLaunchKernelGGL((stream_add_kernel<bf16_t>), grid, block, 0, stream, x,
+                       (const bf16_t*)delta, n_partials, (size_t)partial_stride, origin, vec,
+                       width, total);
+  else
+    return ZA_ERR_UNSUPPORTED;
+  return za_launch_status();
 }
 
 extern "C" int za_embed_gather(const int* tokens, const void* table, int table_dtype, float* out,

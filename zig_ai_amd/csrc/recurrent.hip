@@ -17,6 +17,9 @@
 //          g = exp(-exp(A_log) * softplus(raw + dt_bias))   (one per head and key channel)
 //          q, k made unit vectors (x / sqrt(sum x^2 + 1e-6)), q times dk^(-1/2),
 //          beta = sigmoid(raw)
+//      fixed decay (retention):      S <- a_h S + k v^T;             o = S^T q
+//          a_h a constant of the head; the SSD walk with dt = 1 and no D, q and k rotated
+//          and k scaled beforehand by retention_prepare
 //    A column of S never meets another column: P neighbouring lanes that split its rows
 //    keep one column in registers across all tokens of the portion, read it from the
 //    slot at the start and store it at the end.  The slot holds S turned round,
@@ -32,6 +35,7 @@
 #include <math.h>
 
 #include "common.h"
+#include "rope_math.h"
 
 #define RC_MAX_TAPS 8
 
@@ -174,6 +178,8 @@ struct RecurrenceArgs {
   const int* slot_id;
   float* out;             // [T][H*dv] 32-bit
   int H, G, dk, dv;
+  const float* fixed_decay;   // [H], or null: the SSD walk with this decay, dt = 1 and no
+                              // raw step sizes (proj, dt_bias, A_log are not read then)
 };
 
 // Everything of a token that does not depend on the state, for the delta rule: the unit
@@ -316,9 +322,11 @@ matrix_recurrence_kernel(RecurrenceArgs a) {
         if (part * R + r < dk) S[r] = st[r];
     }
   }
-  const float neg_A = DELTA ? 0.f : -expf(a.A_log[h]);
-  const float Dh = DELTA ? 0.f : a.D[h];
-  const float dtb = DELTA ? 0.f : a.dt_bias[h];
+  const bool fixed = !DELTA && a.fixed_decay != nullptr;
+  const float fixed_a = fixed ? a.fixed_decay[h] : 0.f;
+  const float neg_A = (DELTA || fixed) ? 0.f : -expf(a.A_log[h]);
+  const float Dh = (DELTA || !a.D) ? 0.f : a.D[h];
+  const float dtb = (DELTA || fixed) ? 0.f : a.dt_bias[h];
 
   // (whole four-float loads need the vectors to start on 16-byte boundaries)
   bool vec_loads = dk % 4 == 0 && stride % 4 == 0;
@@ -360,7 +368,7 @@ matrix_recurrence_kernel(RecurrenceArgs a) {
       const size_t t = start + c0 + lane;
       if (DELTA) {
         snext = a.prep[t * a.prep_width + 2 * a.G * dk + a.H * dk + h];
-      } else {
+      } else if (!fixed) {
         const size_t at = t * a.proj_stride + a.gate_col + h;
         snext = a.proj_bf16 ? (float)((const bf16_t*)a.proj)[at] : ((const float*)a.proj)[at];
       }
@@ -378,8 +386,8 @@ matrix_recurrence_kernel(RecurrenceArgs a) {
       if (DELTA) {
         scal[buf][lane][0] = snext;
       } else {
-        const float dt = softplus_f(snext + dtb);
-        scal[buf][lane][0] = lane < chunk_left ? expf(neg_A * dt) : 1.f;
+        const float dt = fixed ? 1.f : softplus_f(snext + dtb);
+        scal[buf][lane][0] = lane < chunk_left ? (fixed ? fixed_a : expf(neg_A * dt)) : 1.f;
         scal[buf][lane][1] = lane < chunk_left ? dt : 0.f;
       }
     }
@@ -516,7 +524,8 @@ static int launch_recurrence(const RecurrenceArgs& a, int n_seqs, int P, bool lo
   return za_launch_status();
 }
 
-// `form`: 0 = SSD, 1 = gated delta rule.  `lanes` (P): the power of two, at most 64, with
+// `form`: 0 = SSD, 1 = gated delta rule, 2 = fixed decay (`decay` then holds H 32-bit
+// decays, one per head; proj, dt_bias, A_log and D are not read).  `lanes` (P): the power of two, at most 64, with
 // 16 * P >= dk that splits a column's rows.  `prep` (delta): [n_tokens][prep_width]
 // floats of scratch, prep_width >= 2*G*dk + H*dk + H.
 extern "C" int za_matrix_recurrence(int form, int dtype, const float* conv, int conv_width,
@@ -529,22 +538,27 @@ extern "C" int za_matrix_recurrence(int form, int dtype, const float* conv, int 
                                     int H, int G, int dk, int dv, int lanes,
                                     hipStream_t stream) {
   if (n_seqs == 0 || n_tokens == 0) return 0;
+  if (form < 0 || form > 2) return ZA_ERR_ARG;
   if (n_seqs < 0 || n_tokens < 0 || H <= 0 || G <= 0 || H % G || dk <= 0 || dv <= 0 || !conv ||
-      !proj || !dt_bias || !A_log || !state || !seq_start || !slot_id || !out)
+      !state || !seq_start || !slot_id || !out)
     return ZA_ERR_ARG;
-  if (form == 0 ? !D : (!decay || decay_stride < H * dk || !prep ||
-                        prep_width < 2 * G * dk + H * dk + H))
+  if (form != 2 && (!proj || !dt_bias || !A_log)) return ZA_ERR_ARG;
+  if (form == 2 && !decay) return ZA_ERR_ARG;
+  if (form == 0 && !D) return ZA_ERR_ARG;
+  if (form == 1 && (!decay || decay_stride < H * dk || !prep ||
+                    prep_width < 2 * G * dk + H * dk + H))
     return ZA_ERR_ARG;
   if (lanes < 1 || lanes > 64 || (lanes & (lanes - 1)) || lanes * RC_ROWS < dk ||
       slot_stride < (long long)H * dk * dv)
     return ZA_ERR_ARG;
   if (dtype != 0 && dtype != 1) return ZA_ERR_UNSUPPORTED;
   RecurrenceArgs a{conv, conv_width, q_col, k_col, x_col, proj, proj_stride, gate_col, dtype,
-                   prep, prep_width, dt_bias, A_log, D, state, slot_stride, seq_start, slot_id,
-                   out, H, G, dk, dv};
+                   prep, prep_width, dt_bias, A_log, form == 2 ? nullptr : D, state, slot_stride,
+                   seq_start, slot_id, out, H, G, dk, dv,
+                   form == 2 ? (const float*)decay : nullptr};
   // (a function of the step's shape alone, as a recorded step needs it)
   const bool long_portions = n_tokens > 4 * n_seqs;
-  if (form == 0) return launch_recurrence<false>(a, n_seqs, lanes, long_portions, stream);
+  if (form != 1) return launch_recurrence<false>(a, n_seqs, lanes, long_portions, stream);
   const dim3 prep_grid(n_tokens, 2 * G + (H * dk + 255) / 256);
   if (dtype == 0)
     hipLaunchKernelGGL((delta_prepare_kernel<float>), prep_grid, dim3(64), 0, stream, conv,
@@ -559,6 +573,67 @@ extern "C" int za_matrix_recurrence(int form, int dtype, const float* conv, int 
   const int rc = za_launch_status();
   if (rc != 0) return rc;
   return launch_recurrence<true>(a, n_seqs, lanes, long_portions, stream);
+}
+
+// ------------------------------------------------------------ retention's vectors
+// What the fixed-decay walk reads, from the opening projection's rows: per token the
+// queries and keys of every head with the first `rot` elements of each rotated by the
+// token's position (element i paired with i + rot/2, angle = position * inv_freq[i]) and
+// the keys times `k_scale`, then the values, all as 32-bit floats:
+//   prep[t] = [q: H*dk | k: H*dk | v: H*dv]
+// grid (tokens, heads), one wave.
+template <typename T>
+__global__ void __launch_bounds__(64)
+retention_prepare_kernel(const T* __restrict__ proj, int proj_stride, int q_col, int k_col,
+                         int v_col, const int* __restrict__ positions,
+                         const float* __restrict__ inv_freq, float* __restrict__ prep, int H,
+                         int dk, int dv, int rot, float k_scale) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const T* row = proj + (size_t)t * proj_stride;
+  float* dst = prep + (size_t)t * (2 * H * dk + H * dv);
+  const int pos = positions[t], half = rot / 2;
+  for (int i = lane; i < dk; i += 64) {
+    const float q = to_f32<T>(row[q_col + h * dk + i]);
+    const float k = to_f32<T>(row[k_col + h * dk + i]);
+    float qo = q, ko = k;
+    if (i < rot) {
+      const bool low = i < half;
+      const int j = low ? i : i - half, partner = low ? i + half : i - half;
+      float cs, sn;
+      rope_angle(pos, inv_freq[j], &cs, &sn);
+      const float qp = to_f32<T>(row[q_col + h * dk + partner]);
+      const float kp = to_f32<T>(row[k_col + h * dk + partner]);
+      qo = low ? rope_rotate_low(q, qp, cs, sn) : rope_rotate_high(q, qp, cs, sn);
+      ko = low ? rope_rotate_low(k, kp, cs, sn) : rope_rotate_high(k, kp, cs, sn);
+    }
+    dst[h * dk + i] = qo;
+    dst[H * dk + h * dk + i] = ko * k_scale;
+  }
+  for (int i = lane; i < dv; i += 64)
+    dst[2 * H * dk + h * dv + i] = to_f32<T>(row[v_col + h * dv + i]);
+}
+
+extern "C" int za_retention_prepare(const void* proj, int dtype, int proj_stride, int q_col,
+                                    int k_col, int v_col, const int* positions,
+                                    const float* inv_freq, float* prep, int n_tokens, int H, int dk,
+                                    int dv, int rot, float k_scale, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  if (n_tokens < 0 || H <= 0 || dk <= 0 || dv <= 0 || !proj || !positions || !prep || rot < 0 ||
+      rot > dk || rot % 2 || (rot > 0 && !inv_freq) || q_col < 0 || k_col < 0 || v_col < 0 ||
+      q_col + H * dk > proj_stride || k_col + H * dk > proj_stride || v_col + H * dv > proj_stride)
+    return ZA_ERR_ARG;
+  dim3 grid(n_tokens, H), block(64);
+  if (dtype == 0)
+    hipLaunchKernelGGL((retention_prepare_kernel<float>), grid, block, 0, stream,
+                       (const float*)proj, proj_stride, q_col, k_col, v_col, positions, inv_freq,
+                       prep, H, dk, dv, rot, k_scale);
+  else if (dtype == 1)
+    hipLaunchKernelGGL((retention_prepare_kernel<bf16_t>), grid, block, 0, stream,
+                       (const bf16_t*)proj, proj_stride, q_col, k_col, v_col, positions, inv_freq,
+                       prep, H, dk, dv, rot, k_scale);
+  else
+    return ZA_ERR_UNSUPPORTED;
+  return za_launch_status();
 }
 
 // ------------------------------------------------------------- gated group norm

@@ -100,6 +100,11 @@ class DecoderModel:
                 note(p)
             self.blocks.append(arrangement(built, **dict(getattr(layer, "params", None) or {})))
             self.mixer_slots.append([n for n, family in slots.items() if family == "mixer"])
+        # what enters the stream between run-order entries (``LayerCall.before``)
+        self.stream_parts = [make("stream", part, ("stream", i))
+                             for i, part in enumerate(getattr(spec, "stream_parts", ()))]
+        for p in self.stream_parts:
+            note(p)
         self.final_norm = make("norm", spec.final_norm, ("final_norm",))
         self.head = make("head", spec.lm_head, ("lm_head",))
         note(self.final_norm)
@@ -129,7 +134,7 @@ class DecoderModel:
                 if self.cache_needs[key] is not None and key not in writers:
                     raise ValueError(f"cache {key} is read but no run-order entry writes it")
         # (what a part holds inside it, a mixer's position encoding for one, is asked too)
-        top = [self.embedding, self.final_norm, self.head]
+        top = [self.embedding, self.final_norm, self.head] + list(self.stream_parts)
         for b in self.blocks:
             top += list(b.parts.values())
         every = [q for p in top for q in walk_parts(p)]
@@ -194,7 +199,7 @@ class DecoderModel:
             stored = random_tensor(seed, exp.names[0], exp.rule.stored_shape or exp.rule.shapes[0],
                                    exp.rule.role, rt.dtype,
                                    deviation_of(exp.names[0], exp.rule.role, std, role_std or {}),
-                                   norm_init, device, quick=quick)
+                                   norm_init, device, quick=quick, bound=exp.rule.bound)
             kept = keep_dtype(stored.dtype, exp.rule.role, rt.dtype)
             tensors.setdefault(exp.owner, {})[exp.local] = \
                 stored.reshape(exp.rule.shapes[0]).to(kept).contiguous()
@@ -247,8 +252,14 @@ class DecoderModel:
         pending = None
         if taps is not None:
             taps.append({"stream": residual.clone()})
+        # (the stream is updated in place: what may ask for the embedding's output later
+        # gets a copy of it)
+        origin = residual.clone() if any(c.before is not None for c in self.schedule) else None
         for call, view in zip(self.schedule, views):
             step.taps = {} if taps is not None else None
+            if call.before is not None:
+                residual, pending = self.stream_parts[call.before.part].forward(
+                    residual, pending, origin, step, **dict(call.before.args))
             residual, pending = self.blocks[call.layer].forward(residual, pending, step, view)
             if taps is not None:
                 now = residual.clone()

@@ -28,7 +28,7 @@ PACKAGE_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC_DIR = os.path.join(PACKAGE_DIR, "csrc")
 ARCH = "gfx950"
 SOURCES = ("norm", "gemm", "gemm_rows64", "rope_kv", "attention", "shortconv", "recurrent",
-           "activation", "sampling", "blaslt", "calibrate")
+           "activation", "experts", "sampling", "blaslt", "calibrate")
 HOST_SOURCES = ("host", "plain")    # plain C++, no device code: usable without a GPU or ROCm
 ALL_SOURCES = SOURCES + HOST_SOURCES
 CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden"]
@@ -40,7 +40,8 @@ HIPCC_FLAGS = [
 
 EXTRA_FLAGS = {"blaslt": ["-lhipblaslt"]}   # host code around the GEMM library, no kernels
 # headers a source includes beside common.h
-EXTRA_HEADERS = {"sampling": ["no_alloc.h"], "rope_kv": ["rope_math.h"], "attention": ["rope_math.h"]}
+EXTRA_HEADERS = {"sampling": ["no_alloc.h"], "rope_kv": ["rope_math.h"], "attention": ["rope_math.h"],
+                 "recurrent": ["rope_math.h"]}
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()

@@ -112,6 +112,26 @@ _SIGNATURES = {
     ("recurrent", "za_gated_group_norm"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int,
                                            c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
                                            c_int, c_int, c_float, c_void_p],
+    ("norm", "za_add_layernorm"): [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                                   c_void_p, c_int, c_int, c_float, c_int, c_int, c_longlong,
+                                   c_void_p],
+    ("norm", "za_stream_add"): [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p,
+                                c_int, c_int, c_void_p],
+    ("activation", "za_gated_unit"): [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    ("activation", "za_scale"): [c_void_p, c_float, c_longlong, c_void_p],
+    ("recurrent", "za_retention_prepare"): [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p,
+                                            c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                            c_float, c_void_p],
+    ("attention", "za_paged_attention_shaped"): [c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                                 c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                                 c_int, c_void_p, c_void_p, c_int, c_int, c_int,
+                                                 c_int, c_int, c_int, c_float, c_int, c_int, c_int,
+                                                 c_float, c_void_p, c_float, c_int, c_void_p],
+    ("experts", "za_expert_lists"): [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
+                                     c_void_p, c_void_p],
+    ("experts", "za_grouped_gemm"): [c_void_p, c_int, c_longlong, c_void_p, c_int, c_void_p,
+                                     c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                     c_int, c_int, c_int, c_float, c_void_p],
 }
 _functions = {}
 
@@ -245,6 +265,77 @@ def embed_gather(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
                                         tokens.numel(), width, vocab, _stream())
     _check(rc, "embed_gather")
     return out
+
+
+def add_layernorm(residual: Optional[torch.Tensor], delta: Optional[torch.Tensor],
+                  weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
+                  out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
+                  write_residual: bool = True) -> torch.Tensor:
+    """``add_rmsnorm`` with the mean taken off first and ``bias`` added last:
+    ``(h - mean) / sqrt(mean((h - mean)^2) + eps) * weight + bias``, ``h = residual + delta``."""
+    if residual is None and delta is None:
+        raise KernelError("add_layernorm needs residual or delta")
+    n_partials, partial_stride = 1, 0
+    if delta is not None and delta.dim() == 3:
+        _need(delta, "delta", torch.float32)
+        n_partials = delta.shape[0]
+        partial_stride = delta.shape[1] * delta.shape[2]
+        shape2 = tuple(delta.shape[1:])
+    else:
+        shape2 = tuple((residual if residual is not None else delta).shape)
+    if len(shape2) != 2:
+        raise KernelError(f"add_layernorm takes [rows, width], got {shape2}")
+    n, width = shape2
+    if residual is not None:
+        _need(residual, "residual", torch.float32, (n, width))
+    if delta is not None and delta.dim() == 2:
+        _need(delta, "delta", (torch.float32, torch.bfloat16), (n, width))
+    _need(weight, "weight", torch.float32, (width,))
+    if bias is not None:
+        _need(bias, "bias", torch.float32, (width,))
+    n_out = n
+    if rows is not None:
+        _need(rows, "rows", torch.int32)
+        n_out = rows.numel()
+    ref = residual if residual is not None else delta
+    out = torch.empty((n_out, width), dtype=out_dtype, device=ref.device)
+    rc = _fn("norm", "za_add_layernorm")(
+        _ptr(residual), _ptr(delta), _code(delta.dtype) if delta is not None else 0, _ptr(weight),
+        _ptr(bias), _ptr(out), _code(out_dtype), _ptr(rows), n_out, width, float(eps),
+        1 if (write_residual and residual is not None and delta is not None and rows is None) else 0,
+        n_partials, partial_stride, _stream())
+    _check(rc, "add_layernorm")
+    return out
+
+
+def stream_add_(stream: torch.Tensor, delta: Optional[torch.Tensor] = None,
+                origin: Optional[torch.Tensor] = None,
+                vector: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``stream [T, width]`` (32-bit, in place) takes ``delta`` (``[T, width]`` of either type
+    or a 32-bit stack ``[P, T, width]`` of partial sums), ``origin`` (32-bit ``[T, width]``)
+    and ``vector`` (32-bit ``[width]``, the same for every row); each may be absent."""
+    _need(stream, "stream", torch.float32)
+    if stream.dim() != 2:
+        raise KernelError(f"stream_add_ takes [rows, width], got {tuple(stream.shape)}")
+    n, width = stream.shape
+    n_partials, partial_stride, code = 1, 0, 0
+    if delta is not None:
+        if delta.dim() == 3:
+            _need(delta, "delta", torch.float32)
+            if tuple(delta.shape[1:]) != (n, width):
+                raise KernelError(f"delta has shape {tuple(delta.shape)}")
+            n_partials, partial_stride = delta.shape[0], n * width
+        else:
+            _need(delta, "delta", (torch.float32, torch.bfloat16), (n, width))
+        code = _code(delta.dtype)
+    if origin is not None:
+        _need(origin, "origin", torch.float32, (n, width))
+    if vector is not None:
+        _need(vector, "vector", torch.float32, (width,))
+    rc = _fn("norm", "za_stream_add")(_ptr(stream), _ptr(delta), code, n_partials, partial_stride,
+                                      _ptr(origin), _ptr(vector), n, width, _stream())
+    _check(rc, "stream_add_")
+    return stream
 
 
 class NormedRows:
@@ -895,15 +986,42 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, positions: torch.Tensor,
 ATTENTION_MAX_ROWS = 32
 
 
+class ScoreShape:
+    """What a design adds to an attention's scores and softmax, for every attention kernel:
+    ``softcap`` (``s <- softcap * tanh(s / softcap)`` after the scale; 0: none), ``sink``
+    (32-bit ``[heads]``: ``exp(sink[h])`` joins the softmax's denominator once, with no key
+    and no value; None: none) and ``temperature`` (``(coef, every)``: the query at position
+    ``p`` counts ``1 + coef * ln(floor((p + 1) / every) + 1)`` times; None: none)."""
+
+    def __init__(self, softcap: float = 0.0, sink: Optional[torch.Tensor] = None,
+                 temperature: Optional[Tuple[float, int]] = None):
+        self.softcap = float(softcap or 0.0)
+        self.sink = sink
+        self.coef, self.every = (float(temperature[0]), int(temperature[1])) if temperature \
+            else (0.0, 0)
+        if self.softcap < 0.0 or self.every < 0:
+            raise KernelError("softcap and the temperature's period must not be negative")
+
+    def args(self, num_heads: int):
+        if self.sink is not None:
+            _need(self.sink, "sink", torch.float32, (num_heads,))
+        return self.softcap, _ptr(self.sink), self.coef, self.every
+
+    def __bool__(self) -> bool:
+        return bool(self.softcap or self.sink is not None or self.every)
+
+
 def paged_attention(q: torch.Tensor, kv_cache: torch.Tensor, block_table: torch.Tensor,
                     positions: torch.Tensor, item_seq: torch.Tensor, item_row0: torch.Tensor,
                     item_count: torch.Tensor, n_items: int, scale: float, window: int = 0,
                     keys_per_split: int = 0, nsplit: int = 1,
-                    workspace: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> torch.Tensor:
+                    workspace: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                    shape: Optional[ScoreShape] = None) -> torch.Tensor:
     """Causal attention of ``q [T, heads, head_dim]`` over the cache; see
     csrc/attention.hip.  ``item_*`` list the work items: the request (row of
     ``block_table``), the first query row and the number of consecutive query
-    rows, at most ``ATTENTION_MAX_ROWS // (heads // kv_heads)`` each."""
+    rows, at most ``ATTENTION_MAX_ROWS // (heads // kv_heads)`` each.  ``shape``: see
+    ``ScoreShape``."""
     if q.dim() != 3:
         raise KernelError(f"q must be [T, heads, head_dim], got {tuple(q.shape)}")
     T, nh, d = q.shape
@@ -942,11 +1060,18 @@ def paged_attention(q: torch.Tensor, kv_cache: torch.Tensor, block_table: torch.
         else:
             part_acc = torch.empty((T, nh, nsplit, d), dtype=torch.float32, device=q.device)
             part_ml = torch.empty((T, nh, nsplit, 2), dtype=torch.float32, device=q.device)
-    rc = _fn("attention", "za_paged_attention")(
-        _ptr(q), _ptr(out), _ptr(kv_cache), _ptr(block_table), block_table.shape[1],
-        _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
-        _ptr(part_acc), _ptr(part_ml), _code(q.dtype), nh, nkv, d, page_size, float(scale),
-        int(window), int(keys_per_split), int(nsplit), _stream())
+    if shape:
+        rc = _fn("attention", "za_paged_attention_shaped")(
+            _ptr(q), _ptr(out), _ptr(kv_cache), _ptr(block_table), block_table.shape[1],
+            _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
+            _ptr(part_acc), _ptr(part_ml), _code(q.dtype), nh, nkv, d, d, page_size, float(scale),
+            int(window), int(keys_per_split), int(nsplit), *shape.args(nh), _stream())
+    else:
+        rc = _fn("attention", "za_paged_attention")(
+            _ptr(q), _ptr(out), _ptr(kv_cache), _ptr(block_table), block_table.shape[1],
+            _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
+            _ptr(part_acc), _ptr(part_ml), _code(q.dtype), nh, nkv, d, page_size, float(scale),
+            int(window), int(keys_per_split), int(nsplit), _stream())
     _check(rc, "paged_attention")
     _note("attention", kernel="plain", rows=T, dtype=q.dtype, nsplit=int(nsplit))
     return out
@@ -1235,6 +1360,33 @@ def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
                                         two_i // 2, _stream())
     _check(rc, "swiglu")
     return out
+
+
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def gated_unit(gate_up: torch.Tensor, activation: str) -> torch.Tensor:
+    """``act(gate) * up`` on a fused ``[T, 2I]`` projection; ``activation``: ``silu`` or
+    ``gelu_tanh`` (0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))), in 32-bit."""
+    if activation not in GATE_ACTIVATIONS:
+        raise KernelError(f"activation must be one of {sorted(GATE_ACTIVATIONS)}, got {activation!r}")
+    _need(gate_up, "gate_up", (torch.float32, torch.bfloat16))
+    if gate_up.dim() != 2 or gate_up.shape[1] % 2:
+        raise KernelError(f"gated_unit takes [T, 2I], got {tuple(gate_up.shape)}")
+    T, inter = gate_up.shape[0], gate_up.shape[1] // 2
+    out = torch.empty((T, inter), dtype=gate_up.dtype, device=gate_up.device)
+    rc = _fn("activation", "za_gated_unit")(_ptr(gate_up), _ptr(out), _code(gate_up.dtype), T,
+                                            inter, GATE_ACTIVATIONS[activation], _stream())
+    _check(rc, "gated_unit")
+    return out
+
+
+def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:
+    """``x *= factor`` for a 32-bit tensor, in place."""
+    _need(x, "x", torch.float32)
+    rc = _fn("activation", "za_scale")(_ptr(x), float(factor), x.numel(), _stream())
+    _check(rc, "scale_")
+    return x
 
 
 def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
@@ -1617,8 +1769,11 @@ def matrix_recurrence(form: str, conv: torch.Tensor, q_col: int, k_col: int, x_c
     ``gate_col`` (ssd: the step size, delta: the write strength); ``decay [T, >= heads*dk]``
     (delta) the raw decays in its first ``heads*dk`` columns.  The state of slot ``s`` lies at ``state[s, state_offset:]`` as
     ``[heads][dv][dk]``.  Returns 32-bit ``[T, heads*dv]``."""
-    if form not in ("ssd", "delta"):
-        raise KernelError(f"form must be ssd or delta, got {form!r}")
+    if form not in ("ssd", "delta", "fixed"):
+        raise KernelError(f"form must be ssd, delta or fixed, got {form!r}")
+    if form == "fixed":
+        return _fixed_decay_recurrence(conv, q_col, k_col, x_col, decay, state, state_offset,
+                                       seq_start, slot_id, heads, groups, dk, dv)
     delta = form == "delta"
     T, conv_width = conv.shape
     _need(conv, "conv", torch.float32)
@@ -1663,6 +1818,66 @@ def matrix_recurrence(form: str, conv: torch.Tensor, q_col: int, k_col: int, x_c
     return out
 
 
+def _fixed_decay_recurrence(vectors: torch.Tensor, q_col: int, k_col: int, x_col: int,
+                            decay: torch.Tensor, state: torch.Tensor, state_offset: int,
+                            seq_start: torch.Tensor, slot_id: torch.Tensor, heads: int, groups: int,
+                            dk: int, dv: int) -> torch.Tensor:
+    """``matrix_recurrence``'s form ``"fixed"``: ``S <- decay[h] S + k v^T; o = S^T q`` with one
+    constant decay a head (32-bit ``[heads]``); ``vectors [T, columns]`` holds q and k
+    (``groups`` of ``dk``) and v (``heads`` of ``dv``) at the three columns."""
+    T, width = vectors.shape
+    _need(vectors, "vectors", torch.float32)
+    _need(decay, "decay", torch.float32, (heads,))
+    if heads % groups:
+        raise KernelError(f"{heads} heads do not divide into {groups} groups")
+    for name, col, n in (("q_col", q_col, groups * dk), ("k_col", k_col, groups * dk),
+                         ("x_col", x_col, heads * dv)):
+        if col < 0 or col + n > width:
+            raise KernelError(f"{name}: columns {col}..{col + n} of {width}")
+    S = slot_id.numel()
+    _need(seq_start, "seq_start", torch.int32, (S + 1,))
+    _need(slot_id, "slot_id", torch.int32, (S,))
+    base, slot_stride = _state_window(state, state_offset, heads * dk * dv, "state")
+    lanes, _, _ = recurrence_plan(dk, dv)
+    out = torch.empty((T, heads * dv), dtype=torch.float32, device=vectors.device)
+    rc = _fn("recurrent", "za_matrix_recurrence")(
+        2, 0, _ptr(vectors), width, int(q_col), int(k_col), int(x_col), None, 0, 0, _ptr(decay),
+        0, None, None, None, None, 0, base, slot_stride, _ptr(seq_start), _ptr(slot_id),
+        _ptr(out), T, S, heads, groups, dk, dv, lanes, _stream())
+    _check(rc, "matrix_recurrence", f"form=fixed heads={heads} dk={dk} dv={dv}")
+    return out
+
+
+def retention_prepare(proj: torch.Tensor, q_col: int, k_col: int, v_col: int,
+                      positions: torch.Tensor, inv_freq: Optional[torch.Tensor], heads: int, dk: int,
+                      dv: int, rotary_dim: int, k_scale: float) -> torch.Tensor:
+    """From an opening projection's rows ``proj [T, columns]`` (queries, keys and values of
+    ``heads`` heads at the three columns) the 32-bit vectors of the fixed-decay recurrence,
+    ``[T, q: heads*dk | k: heads*dk | v: heads*dv]``: the first ``rotary_dim`` elements of
+    every query and key rotated by the token's position (element ``i`` with ``i +
+    rotary_dim/2``, angle ``position * inv_freq[i]``), the keys times ``k_scale``."""
+    _need(proj, "proj", (torch.float32, torch.bfloat16))
+    if proj.dim() != 2:
+        raise KernelError(f"proj must be [T, columns], got {tuple(proj.shape)}")
+    T, stride = proj.shape
+    _need(positions, "positions", torch.int32, (T,))
+    if rotary_dim:
+        _need(inv_freq, "inv_freq", torch.float32, (rotary_dim // 2,))
+    if rotary_dim < 0 or rotary_dim % 2 or rotary_dim > dk:
+        raise KernelError(f"rotary_dim {rotary_dim} must be even and at most {dk}")
+    for name, col, n in (("q_col", q_col, heads * dk), ("k_col", k_col, heads * dk),
+                         ("v_col", v_col, heads * dv)):
+        if col < 0 or col + n > stride:
+            raise KernelError(f"{name}: columns {col}..{col + n} of {stride}")
+    out = torch.empty((T, 2 * heads * dk + heads * dv), dtype=torch.float32, device=proj.device)
+    rc = _fn("recurrent", "za_retention_prepare")(
+        _ptr(proj), _code(proj.dtype), stride, int(q_col), int(k_col), int(v_col), _ptr(positions),
+        _ptr(inv_freq) if rotary_dim else None, _ptr(out), T, heads, dk, dv, int(rotary_dim),
+        float(k_scale), _stream())
+    _check(rc, "retention_prepare")
+    return out
+
+
 def gated_group_norm(y: torch.Tensor, gate: torch.Tensor, gate_col: int, weight: torch.Tensor,
                      group: int, eps: float, activation: str, gate_first: bool,
                      out_scale: float = 1.0) -> torch.Tensor:
@@ -1687,4 +1902,69 @@ def gated_group_norm(y: torch.Tensor, gate: torch.Tensor, gate_col: int, weight:
         weight.numel(), _ptr(out), width, 0, T, width, int(group), float(eps),
         1 if activation == "silu" else 0, 1 if gate_first else 0, float(out_scale), _stream())
     _check(rc, "gated_group_norm")
+    return out
+
+
+# ------------------------------------------------------------------- experts
+EXPERTS_MAX = 1024
+
+
+def expert_lists(ids: Optional[torch.Tensor], table: torch.Tensor, n_tokens: int, experts: int):
+    """Who goes to which expert: ``table [rows, top]`` (int32) names the experts of row
+    ``ids[t]`` (``ids`` int32 ``[T]``; None: row ``t`` itself).  Returns ``(lists [experts, T*top],
+    counts [experts])``, int32: expert ``e``'s assignments ``a = t * top + j`` ascending in
+    ``lists[e, :counts[e]]`` (the rest of a row is not written)."""
+    _need(table, "table", torch.int32)
+    if table.dim() != 2:
+        raise KernelError(f"table must be [rows, top], got {tuple(table.shape)}")
+    rows, top = table.shape
+    if ids is not None:
+        _need(ids, "ids", torch.int32, (n_tokens,))
+    elif rows < n_tokens:
+        raise KernelError(f"a table of {rows} rows for {n_tokens} tokens")
+    if not 0 < experts <= EXPERTS_MAX:
+        raise KernelError(f"{experts} experts: the kernels take 1 to {EXPERTS_MAX}")
+    lists = torch.empty((experts, n_tokens * top), dtype=torch.int32, device=table.device)
+    counts = torch.empty((experts,), dtype=torch.int32, device=table.device)
+    rc = _fn("experts", "za_expert_lists")(_ptr(ids), _ptr(table), rows, n_tokens, top, experts,
+                                           _ptr(lists), _ptr(counts), _stream())
+    _check(rc, "expert_lists")
+    return lists, counts
+
+
+EXPERT_ACTIVATIONS = {None: 0, "relu2": 1}
+
+
+def grouped_linear(src: torch.Tensor, weights: torch.Tensor, lists: torch.Tensor,
+                   counts: torch.Tensor, n_tokens: int, per_token: bool, stacked: bool = False,
+                   activation: Optional[str] = None, out_scale: float = 1.0,
+                   out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """Every assignment's row times its expert's weight: ``weights [experts, N, K]``,
+    ``src [T, K]`` (``per_token``: assignment ``a`` reads row ``a // top``) or ``[T*top, K]``
+    (one row an assignment).  Returns ``[T*top, N]`` in assignment order, or with ``stacked``
+    32-bit ``[top, T, N]``: a stack of partial results that ``add_rmsnorm`` /
+    ``add_layernorm`` / ``stream_add_`` add up.  ``activation``: None or ``relu2`` (the square
+    of relu), applied before ``out_scale``."""
+    if activation not in EXPERT_ACTIVATIONS:
+        raise KernelError(f"activation must be None or relu2, got {activation!r}")
+    _need(weights, "weights", (torch.float32, torch.bfloat16))
+    if weights.dim() != 3:
+        raise KernelError(f"weights must be [experts, N, K], got {tuple(weights.shape)}")
+    E, N, K = weights.shape
+    _need(lists, "lists", torch.int32)
+    _need(counts, "counts", torch.int32, (E,))
+    if lists.dim() != 2 or lists.shape[0] != E or n_tokens <= 0 or lists.shape[1] % n_tokens:
+        raise KernelError(f"lists has shape {tuple(lists.shape)} for {E} experts and {n_tokens} tokens")
+    top = lists.shape[1] // n_tokens
+    _need(src, "src", (torch.float32, torch.bfloat16), (n_tokens if per_token else n_tokens * top, K))
+    if weights.dtype == torch.bfloat16 and (src.dtype != torch.bfloat16 or K % 8):
+        raise KernelError("bfloat16 expert weights need bfloat16 rows and K a multiple of 8")
+    out_dtype = torch.float32 if stacked else (out_dtype or src.dtype)
+    shape = (top, n_tokens, N) if stacked else (n_tokens * top, N)
+    out = torch.empty(shape, dtype=out_dtype, device=src.device)
+    rc = _fn("experts", "za_grouped_gemm")(
+        _ptr(src), _code(src.dtype), src.shape[0], _ptr(weights), _code(weights.dtype), _ptr(lists),
+        _ptr(counts), _ptr(out), _code(out_dtype), n_tokens, top, E, N, K, top if per_token else 1,
+        1 if stacked else 0, EXPERT_ACTIVATIONS[activation], float(out_scale), _stream())
+    _check(rc, "grouped_linear", f"E={E} N={N} K={K} tokens={n_tokens} top={top}")
     return out

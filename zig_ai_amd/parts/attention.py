@@ -18,6 +18,15 @@ attention's output per head, of another width than queries and keys) and ``gate`
 (``"head"``: every head's output is multiplied by ``sigmoid(x Wg^T)_h`` before the output
 projection; the gate's rows ride along in the opening projection).  With either, the
 cache is a plane of keys and a plane of values per page.
+
+And what a design may do to the scores (``ops.ScoreShape``; every attention kernel takes
+it): ``softcap`` (``s <- softcap * tanh(s / softcap)`` after the scale), ``sink`` (true: a
+tensor ``sink [num_heads]`` whose exponential joins each head's softmax denominator once,
+with no key and no value) and ``query_temperature`` (``(coef, every)``: the query at
+position ``p`` is multiplied by ``1 + coef * ln(floor((p + 1) / every) + 1)``).
+``values="keys"``: there is no value projection, a token's value is its key as projected
+(the key rows of the opening projection are there a second time, so whatever stores
+q | k | v rows finds the same numbers in the value columns).
 """
 
 from __future__ import annotations
@@ -81,6 +90,10 @@ class GroupedQueryAttention(Mixer):
                  "k_proj.weight": TensorRule(((nkv * d, H),)),
                  "v_proj.weight": TensorRule(((nkv * dv, H),)),
                  "out_proj.weight": TensorRule(((H, nh * dv),))}
+        if params.get("values") == "keys":
+            del rules["v_proj.weight"]
+        if params.get("sink"):
+            rules["sink"] = TensorRule(((nh,),), role="bias")
         if params.get("gate") == "head":
             rules["gate_proj.weight"] = TensorRule(((nh, H),))
         if params.get("qk_norm"):
@@ -139,7 +152,17 @@ class GroupedQueryAttention(Mixer):
         self.item_granularities = [self.rows_per_item] + (
             [self.mfma_rows_per_item, self.mfma_decode_rows_per_item] if self.mfma else [])
         self.eps = float(params.get("norm_eps", 0.0))
-        opening = [tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]]
+        if params.get("values") not in (None, "own", "keys"):
+            raise ValueError(f"attention values must be 'own' or 'keys', got {params.get('values')!r}")
+        self.shared_values = params.get("values") == "keys"
+        if self.shared_values and (self.value_dim != self.head_dim or params.get("bias")):
+            raise ValueError("values that are the keys have the keys' width and no bias")
+        temperature = params.get("query_temperature")
+        self.shape = ops.ScoreShape(params.get("softcap") or 0.0,
+                                    tensors["sink"] if params.get("sink") else None,
+                                    tuple(temperature) if temperature else None)
+        opening = [tensors["q_proj.weight"], tensors["k_proj.weight"],
+                   tensors["k_proj.weight" if self.shared_values else "v_proj.weight"]]
         self.gate_col = (self.num_heads + self.num_kv_heads) * self.head_dim \
             + self.num_kv_heads * self.value_dim
         if self.gated:
@@ -168,7 +191,10 @@ class GroupedQueryAttention(Mixer):
         if self.wide and self.position is not None and not self.fused_rotation:
             raise ValueError("an attention with value_dim or gate takes a rotary position "
                              "encoding or none")
-        self.mfma = self.mfma and self.value_dim == self.head_dim
+        self.mfma = self.mfma and self.value_dim == self.head_dim and not self.shape
+        if self.shape and self.wide:
+            raise ValueError("a cap, a sink or a query temperature go with values of the keys' "
+                             "width and no gate")
         self.rotation_in_attention = (
             not self.wide and self.fused_rotation and runtime.dtype == torch.bfloat16
             and self.position.rotary_dim == self.head_dim and self.position.pairing != "adjacent")
@@ -255,7 +281,7 @@ class GroupedQueryAttention(Mixer):
             keys, nsplit = plan_split(n_items, nkv, step.max_keys)
             o = ops.paged_attention(q, cache.kv, step.block_tables[cache.group], step.positions,
                                     item_seq, item_row0, item_count, n_items, self.scale,
-                                    self.window, keys, nsplit)
+                                    self.window, keys, nsplit, shape=self.shape)
         if getattr(step, "taps", None) is not None:
             self._leave_taps(step, cache, q, o)
         return ops.linear(o.view(T, nh * d), self.w_out, self.b_out, partial_ok=True,

@@ -9,6 +9,8 @@ never learns which model it is in.  Five families exist:
                      (``y`` is ``[T, width]`` or a stack ``[P, T, width]`` of 32-bit
                      partial sums that the following norm adds up)
   norm               ``forward(x) -> y`` and ``add_forward(residual, delta) -> y``
+  stream step        ``forward(residual, pending, origin, step, **args) -> (residual, pending)``:
+                     something that enters the stream between two run-order entries
   position encoding  used by mixers: a rotation table, or ``apply(q, k, positions)``
   arrangement        wires a block's parts (it declares their names and families;
                      two norms, a mixer and a feed-forward in the usual block)
@@ -43,6 +45,9 @@ class TensorRule:
     role: str = "matrix"
     required: bool = True
     stored_shape: Optional[Tuple[int, ...]] = None
+    # role ``choice``: an integer table whose entries lie in [0, bound) and differ within
+    # a row (which of ``bound`` things each row picks); kept as int32
+    bound: int = 0
 
 
 # ---------------------------------------------------------------- cache needs
@@ -207,7 +212,7 @@ class PositionEncoding(Part):
 # ---------------------------------------------------------------- registries
 _REGISTRIES: Dict[str, Dict[str, Any]] = {
     "mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "arrangement": {},
-    "embedding": {}, "head": {},
+    "embedding": {}, "head": {}, "stream": {},
 }
 
 
@@ -242,6 +247,10 @@ def register_embedding(kind: str, cls: Any) -> Any:
 
 def register_head(kind: str, cls: Any) -> Any:
     return _register("head", kind, cls)
+
+
+def register_stream_step(kind: str, cls: Any) -> Any:
+    return _register("stream", kind, cls)
 
 
 def lookup(family: str, kind: str) -> Any:

@@ -62,6 +62,25 @@ def apply_normed(norm, part, residual: torch.Tensor, pending: Optional[torch.Ten
 register_arrangement(PreNormResidualBlock.kind, PreNormResidualBlock)
 
 
+class PreNormMixerBlock:
+    """The pre-norm block of a layer that has no feed-forward: ``y = x + mixer(norm1(x))``."""
+
+    kind = "pre_norm_residual_no_ff"
+    slots = {"mixer_norm": "norm", "mixer": "mixer"}
+
+    def __init__(self, parts):
+        self.parts = dict(parts)
+        self.mixer_norm = parts["mixer_norm"]
+        self.mixer = parts["mixer"]
+
+    def forward(self, residual: torch.Tensor, pending: Optional[torch.Tensor], step,
+                cache) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+        return residual, apply_normed(self.mixer_norm, self.mixer, residual, pending, step, cache)
+
+
+register_arrangement(PreNormMixerBlock.kind, PreNormMixerBlock)
+
+
 class ScaledResidualBlock:
     """A pre-norm block whose parts enter the stream with weights, and which may run two
     mixers side by side on the same normed input and may lack the feed-forward:

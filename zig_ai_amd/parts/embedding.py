@@ -37,7 +37,7 @@ class LinearHead(Part):
     kind = "linear_head"
     graph_safe = True
     takes_stream = True       # ``forward`` accepts a norm that has not run yet
-    kernel_sources = ("gemm",)
+    kernel_sources = ("gemm", "activation")
 
     @classmethod
     def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:
@@ -50,12 +50,17 @@ class LinearHead(Part):
         super().__init__(params, tensors, runtime)
         self.tied = bool(params.get("tied"))
         self.weight = tensors.get("weight")   # the model hands a tied head the embedding table
+        # a constant factor on the logits (1: none)
+        self.logit_scale = float(params.get("logit_scale", 1.0))
 
     def forward(self, x) -> torch.Tensor:
         if not self.tied and self.weight.dtype == torch.bfloat16 and self.weight.shape[1] % 8:
             self.weight = ops.projection_weight(self.weight)     # kept in 32-bit from now on
         ops.check_projection_weight(self.weight, "output head")
-        return ops.linear(x, self.weight, out_dtype=torch.float32, tune=self.runtime.tune)
+        logits = ops.linear(x, self.weight, out_dtype=torch.float32, tune=self.runtime.tune)
+        if self.logit_scale != 1.0:
+            ops.scale_(logits, self.logit_scale)
+        return logits
 
 
 register_embedding(TokenEmbedding.kind, TokenEmbedding)

@@ -56,10 +56,26 @@ class SwiGLU(FeedForward):
         super().__init__(params, tensors, runtime)
         self.gate_up = fuse_rows(tensors["gate.weight"], tensors["up.weight"])
         self.down = tensors["down.weight"]
+        # the gate's activation: ``silu`` (SwiGLU) or ``gelu_tanh`` (the tanh form of gelu);
+        # the products that apply the gate to their own sums know silu only
+        self.activation = str(params.get("activation", "silu"))
+        if self.activation not in ops.GATE_ACTIVATIONS:
+            raise ValueError(f"feed-forward activation must be one of "
+                             f"{sorted(ops.GATE_ACTIVATIONS)}, got {self.activation!r}")
+        if self.activation != "silu":
+            self.opens_with_swiglu = False
+            self.gate_up = ops.projection_weight(self.gate_up)
+            self.down = ops.projection_weight(self.down)
         ops.check_projection_weight(self.gate_up, "feed_forward gate_up")
         ops.check_projection_weight(self.down, "feed_forward down")
 
     def forward(self, x, step=None, stream: Optional[torch.Tensor] = None):
+        if self.activation != "silu":
+            if isinstance(x, ops.NormedRows):
+                x = x.materialise()
+            a = ops.gated_unit(ops.linear(x, self.gate_up, tune=self.runtime.tune), self.activation)
+            return ops.linear(a, self.down, partial_ok=True, accumulate=stream,
+                              tune=self.runtime.tune)
         bf16 = x.dtype == torch.bfloat16 and self.gate_up.dtype == torch.bfloat16
         if bf16 and x.shape[0] <= 16 and x.shape[1] <= 8192:
             # a decode batch: the gate is applied to the projection's accumulators

@@ -63,4 +63,45 @@ class RMSNorm(Norm):
         return ops.NormedRows(residual, self.weight, self.eps, self.runtime.dtype, rows)
 
 
+class LayerNorm(Norm):
+    """``(x - mean) / sqrt(mean((x - mean)^2) + eps) * weight + bias`` in 32-bit; ``bias`` may
+    be left out (``params["bias"] = False``).  ``add_forward`` fuses the residual add, and
+    the sum of a stack of partial results, as the RMS norm's does."""
+
+    kind = "layer_norm"
+    graph_safe = True
+    kernel_sources = ("norm",)
+
+    @classmethod
+    def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:
+        width = int(params["width"])
+        rules = {"weight": TensorRule(((width,),), role="norm")}
+        if params.get("bias", True):
+            rules["bias"] = TensorRule(((width,),), role="bias")
+        return rules
+
+    def __init__(self, params, tensors, runtime: Runtime):
+        super().__init__(params, tensors, runtime)
+        self.width = int(params["width"])
+        self.eps = float(params["eps"])
+        self.weight = tensors["weight"]
+        self.bias = tensors.get("bias") if params.get("bias", True) else None
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        shape = x.shape
+        x2 = x.reshape(-1, shape[-1])
+        if x2.dtype == torch.float32:
+            out = ops.add_layernorm(x2, None, self.weight, self.bias, self.eps, self.runtime.dtype,
+                                    write_residual=False)
+        else:
+            out = ops.add_layernorm(None, x2, self.weight, self.bias, self.eps, self.runtime.dtype)
+        return out.view(shape)
+
+    def add_forward(self, residual: torch.Tensor, delta: Optional[torch.Tensor],
+                    rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return ops.add_layernorm(residual, delta, self.weight, self.bias, self.eps,
+                                 self.runtime.dtype, rows=rows)
+
+
 register_norm(RMSNorm.kind, RMSNorm)
+register_norm(LayerNorm.kind, LayerNorm)

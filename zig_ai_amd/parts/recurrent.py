@@ -23,6 +23,18 @@ channel, shared by the heads), times ``sigmoid(W_g2 W_g1 h)``, and the output pr
 
 Both keep, per request, the state matrix in 32-bit and the convolution's last
 ``kernel_size - 1`` inputs, in one state slot: ``[conv inputs | S]``.
+
+``retention`` (linear attention with one fixed decay a head, no softmax and no
+denominator).  Projections q, k (``num_heads x head_dim``), v and a gate g (``num_heads x
+value_dim``), no biases, no convolution; the position encoding (``position``, a nested
+rotary spec or None) turns the leading elements of every q and k, the keys are then
+multiplied by ``head_dim^-1/2``; per head ``h``
+
+    S <- decay[h] S + k v^T;   o = S^T q
+
+then each head's ``o`` over its root mean square (``norm_eps``, no weight), times
+``silu(g)``, and the output projection.  ``decay`` is a tuple of constants, one a head.
+The state slot holds ``S`` in 32-bit; what enters the walk (rotated q and k, v) is 32-bit.
 """
 
 from __future__ import annotations
@@ -32,7 +44,7 @@ from typing import Any, Dict, Mapping
 import torch
 
 from ..kernels import ops
-from .base import Mixer, Runtime, StateNeed, TensorRule, register_mixer
+from .base import Mixer, Runtime, StateNeed, TensorRule, lookup, register_mixer
 from .feed_forward import fuse_rows, pad_columns, pad_rows
 
 
@@ -191,5 +203,76 @@ class GatedDeltaRule(Mixer):
         return ops.linear(h, self.w_out, tune=self.runtime.tune)
 
 
+class Retention(Mixer):
+    kind = "retention"
+    graph_safe = True
+    takes_normed_rows = True      # ``x`` is only ever handed to ``ops.linear``
+    kernel_sources = ("gemm", "recurrent")
+
+    @staticmethod
+    def _sizes(params):
+        return tuple(int(params[k]) for k in ("hidden_size", "num_heads", "head_dim", "value_dim"))
+
+    @classmethod
+    def tensor_rules(cls, params: Mapping[str, Any]) -> Dict[str, TensorRule]:
+        W, H, d, dv = cls._sizes(params)
+        return {"q_proj.weight": TensorRule(((H * d, W),)),
+                "k_proj.weight": TensorRule(((H * d, W),)),
+                "v_proj.weight": TensorRule(((H * dv, W),)),
+                "gate_proj.weight": TensorRule(((H * dv, W),)),
+                "out_proj.weight": TensorRule(((W, H * dv),))}
+
+    @classmethod
+    def cache_need(cls, params: Mapping[str, Any]):
+        W, H, d, dv = cls._sizes(params)
+        return StateNeed((H * d * dv,))
+
+    def __init__(self, params, tensors, runtime: Runtime):
+        super().__init__(params, tensors, runtime)
+        W, H, d, dv = self._sizes(params)
+        decay = [float(x) for x in params["decay"]]
+        if len(decay) != H:
+            raise ValueError(f"{len(decay)} decays for {H} heads")
+        ops.recurrence_plan(d, dv)
+        self.heads, self.head_dim, self.value_dim = H, d, dv
+        self.eps = float(params["norm_eps"])
+        self.decay = torch.tensor(decay, dtype=torch.float32, device=runtime.device)
+        self.k_scale = float(d) ** -0.5
+        pos = params.get("position")
+        self.position = lookup("position", pos.kind)(pos.params, {}, runtime) if pos is not None \
+            else None
+        if self.position is not None and not (getattr(self.position, "fused_rotation", False)
+                                               and self.position.pairing == "half"):
+            raise ValueError("retention takes a rotary position encoding in halves, or none")
+        self.rotary_dim = self.position.rotary_dim if self.position is not None else 0
+        # one opening product: q | k | v | g
+        self.w_in = ops.projection_weight(pad_rows(fuse_rows(
+            tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"],
+            tensors["gate_proj.weight"])))
+        self.w_out = ops.projection_weight(tensors["out_proj.weight"])
+        self.gate_col = 2 * H * d + H * dv
+        self.ones = torch.ones((1,), dtype=torch.float32, device=runtime.device)
+        ops.check_projection_weight(self.w_in, "retention opening projection")
+        ops.check_projection_weight(self.w_out, "retention out_proj")
+
+    def forward(self, x, step, cache):
+        H, d, dv = self.heads, self.head_dim, self.value_dim
+        z = ops.linear(x, self.w_in, tune=self.runtime.tune)
+        vectors = ops.retention_prepare(
+            z, 0, H * d, 2 * H * d, step.positions,
+            self.position.inv_freq if self.rotary_dim else None, H, d, dv, self.rotary_dim,
+            self.k_scale)
+        o = ops.matrix_recurrence("fixed", vectors, 0, H * d, 2 * H * d, None, 0, self.decay, None,
+                                  None, None, cache.state, 0, step.seq_start, step.slot_id, H, H,
+                                  d, dv)
+        if getattr(step, "taps", None) is not None:
+            step.taps["vectors"] = vectors.clone()
+            step.taps["o"] = o.clone()
+        h = ops.gated_group_norm(o, z, self.gate_col, self.ones, dv, self.eps, "silu",
+                                 gate_first=False)
+        return ops.linear(h, self.w_out, tune=self.runtime.tune)
+
+
 register_mixer(StateSpaceDuality.kind, StateSpaceDuality)
+register_mixer(Retention.kind, Retention)
 register_mixer(GatedDeltaRule.kind, GatedDeltaRule)

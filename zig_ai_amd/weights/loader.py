@@ -80,6 +80,8 @@ def expected_tensors(spec: ModelSpec) -> List[Expected]:
                 raise KeyError(f"layer {i}: arrangement {layer.arrangement!r} wires a part "
                                f"{name!r} that the layer's description does not give")
             out += _part_expectations(("layer", i, name), family, layer.parts[name])
+    for i, part in enumerate(getattr(spec, "stream_parts", ())):
+        out += _part_expectations(("stream", i), "stream", part)
     out += _part_expectations(("final_norm",), "norm", spec.final_norm)
     out += _part_expectations(("lm_head",), "head", spec.lm_head)
     return out

@@ -87,14 +87,28 @@ def keyed_normal(seed: int, name: str, numel: int, device="cpu",
     return out
 
 
+def random_choices(seed: int, name: str, shape, bound: int, device="cpu") -> torch.Tensor:
+    """An integer table ``[rows, picks]`` (int32) whose rows each hold ``picks`` different
+    numbers below ``bound``: the places of the ``picks`` largest of ``bound`` keyed deviates
+    a row, in the order of their size."""
+    rows, picks = int(shape[0]), int(shape[1])
+    if not 0 < picks <= bound:
+        raise ValueError(f"{name}: {picks} different numbers below {bound}")
+    noise = keyed_normal(seed, name, rows * bound, device).reshape(rows, bound)
+    return torch.argsort(noise, dim=1, descending=True, stable=True)[:, :picks] \
+        .to(torch.int32).contiguous()
+
+
 def random_tensor(seed: int, name: str, shape, role: str, dtype: torch.dtype, std: float,
-                  norm_init: str, device="cpu", quick: bool = False) -> torch.Tensor:
+                  norm_init: str, device="cpu", quick: bool = False, bound: int = 0) -> torch.Tensor:
     """One tensor of a random model: N(0, std) from ``keyed_normal``; norm weights are 1,
     N(0, std) or 1 + N(0, std) by ``norm_init``.  Drawn in 32-bit, rounded to ``dtype``.
     ``quick``: the deviates come from the tensor library's own generator instead, one
     kernel a tensor (seeded by seed and name, but NOT the values a model folder of this
     seed holds): for runs under a profiler's counters, which run every kernel alone, and
     the keyed generator is some hundred small kernels per 16 million values."""
+    if role == "choice":
+        return random_choices(seed, name, shape, bound, device)
     n = 1
     for d in shape:
         n *= int(d)
@@ -149,7 +163,7 @@ def random_tensors(spec, seed: int, dtype: torch.dtype = torch.bfloat16, std: fl
         shape = exp.rule.stored_shape or exp.rule.shapes[0]
         out[name] = random_tensor(seed, name, shape, exp.rule.role, dtype,
                                   deviation_of(name, exp.rule.role, std, role_std), norm_init,
-                                  device).cpu()
+                                  device, bound=exp.rule.bound).cpu()
     return out
 
 
