@@ -54,6 +54,21 @@ __device__ __forceinline__ float capped_score(const ScoreExtras& ex, float s) {
   return ex.softcap > 0.f ? ex.softcap * tanhf(s / ex.softcap) : s;
 }
 
+#define ZA_LOG2E 1.44269504088896341f
+
+// The same for the matrix-core kernels, whose softmax runs on the base-2 scale: the score
+// `dot * row_mul` (row_mul: scale times the row's temperature), capped, times log2(e).
+// tanh(x) = 1 - 2 / (exp(2x) + 1) with the hardware's exp2 and reciprocal: an absolute
+// error of some 1e-7 in tanh, far below what rounding the probabilities to bfloat16 does.
+__device__ __forceinline__ float shaped_score_log2(const ScoreExtras& ex, float dot, float row_mul) {
+  float s = dot * row_mul;
+  if (ex.softcap > 0.f) {
+    const float e = __builtin_amdgcn_exp2f(s * (2.0f * ZA_LOG2E / ex.softcap));
+    s = ex.softcap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f));
+  }
+  return s * ZA_LOG2E;
+}
+
 #define AT_WAVES 4
 #define AT_RPW 8                     // rows per wave, at most
 #define AT_MAX_ROWS (AT_WAVES * AT_RPW)
@@ -350,7 +365,7 @@ __device__ __forceinline__ int page_offset(int kp, int page_size, int shift) {
   return shift >= 0 ? kp & (page_size - 1) : kp % page_size;
 }
 
-template <int D, int NW, int NS, int KT>
+template <int D, int NW, int NS, int KT, bool SHAPED>
 __global__ void __launch_bounds__(NW * 64)
 paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                             const bf16_t* __restrict__ kv, const int* __restrict__ block_table,
@@ -359,7 +374,9 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
                             const int* __restrict__ wi_count, int n_items,
                             float* __restrict__ part_acc, float* __restrict__ part_ml, int nh,
                             int nkv, int page_size, float scale_log2e, int window,
-                            int keys_per_split, int nsplit) {
+                            int keys_per_split, int nsplit, ScoreExtras ex) {
+  // SHAPED: the scores pass `shaped_score_log2` (temperature, cap) and the sink joins the
+  // sum at the end; `ex` is not looked at otherwise
   constexpr int LDK = D + 8;        // padded rows, in elements
   constexpr int LDV = KT + 8;
   constexpr int KSTEPS = D / 32;    // matrix-core steps over the head dimension
@@ -404,6 +421,8 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
   int tok[NS], head[NS], pos_row[NS];
   bool row_valid[NS];
   bf16x8_t qf[NS][KSTEPS];
+  [[maybe_unused]] float row_mul[NS];
+  const float sl2 = SHAPED ? 1.0f : scale_log2e;   // shaped scores are on the base-2 scale already
 #pragma unroll
   for (int c = 0; c < NS; ++c) {
     const int rr = wave * (NS * 16) + c * 16 + r16;
@@ -411,6 +430,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
     tok[c] = row0 + (row_valid[c] ? rr / G : 0);
     head[c] = gkv * G + (row_valid[c] ? rr % G : 0);
     pos_row[c] = row_valid[c] ? positions[tok[c]] : -1;
+    if (SHAPED) row_mul[c] = scale_log2e * (1.0f / ZA_LOG2E) * query_temperature(ex, pos_row[c]);
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks)
       qf[c][ks] = row_valid[c] ? *reinterpret_cast<const bf16x8_t*>(
@@ -556,6 +576,13 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
       bf16x8_t pf[NS][KK];
 #pragma unroll
       for (int c = 0; c < NS; ++c) {
+        if (SHAPED) {
+#pragma unroll
+          for (int jb = 0; jb < JB; ++jb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              s[c][jb][i] = shaped_score_log2(ex, s[c][jb][i], row_mul[c]);
+        }
         if (needs_mask) {
           // key jb * 16 + grp * 4 + i of the tile counts for this lane's row if it lies in
           // [first, last]; both bounds are taken relative to the lane's own keys once, so
@@ -581,7 +608,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
 #pragma unroll
           for (int i = 0; i < 4; ++i) tmax = fmaxf(tmax, s[c][jb][i]);
         tmax = quad_max(tmax);
-        const float m_new = fmaxf(m[c], ceilf(tmax * scale_log2e));   // the factor is positive
+        const float m_new = fmaxf(m[c], ceilf(tmax * sl2));   // the factor is positive
         const float m_use = m_new > -INFINITY ? m_new : 0.f;
         // (nothing is accumulated yet while m is -inf: any finite factor does)
         const float alpha = m[c] > -INFINITY ? ldexpf(1.0f, (int)(m[c] - m_use)) : 1.0f;
@@ -589,7 +616,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
         for (int jb = 0; jb < JB; ++jb)
 #pragma unroll
           for (int i = 0; i < 4; ++i)   // masked scores (-inf) give 0
-            s[c][jb][i] = __builtin_amdgcn_exp2f(fmaf(s[c][jb][i], scale_log2e, -m_use));
+            s[c][jb][i] = __builtin_amdgcn_exp2f(fmaf(s[c][jb][i], sl2, -m_use));
         m[c] = m_new;
         if (__any(alpha != 1.0f)) {
 #pragma unroll
@@ -643,7 +670,10 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
         }
         continue;
       }
-      const float inv = lsum[c][0] > 0.f ? 1.0f / lsum[c][0] : 0.f;
+      float total = lsum[c][0];
+      if (SHAPED && ex.sink && m[c] > -INFINITY)
+        total += exp2f(ex.sink[head[c]] * ZA_LOG2E - m[c]);
+      const float inv = total > 0.f ? 1.0f / total : 0.f;
       bf16_t* dst = out + orow * D;
 #pragma unroll
       for (int db = 0; db < DBLK; ++db) {
@@ -684,7 +714,7 @@ struct DecodeRope {
   int write_kv;
 };
 
-template <int D, int NWV, bool ROPE>
+template <int D, int NWV, bool ROPE, bool SHAPED>
 __global__ void __launch_bounds__(NWV * 64)
 paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                                    const bf16_t* kv,
@@ -694,7 +724,8 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
                                    const int* __restrict__ wi_count, float* __restrict__ part_acc,
                                    float* __restrict__ part_ml, int nh, int nkv, int page_size,
                                    float scale_log2e, int window, int keys_per_split, int nsplit,
-                                   DecodeRope rope) {
+                                   DecodeRope rope, ScoreExtras ex) {
+  // SHAPED: as in paged_attention_mfma_kernel
   constexpr int KSTEPS = D / 32;
   constexpr int DBLK = D / 16;
   __shared__ float mg_m[NWV][16], mg_l[NWV][16];
@@ -855,6 +886,8 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
   const int pos_first = positions[row0];
   const int pos_last = positions[row0 + count - 1];
   const int pos_row = row_valid ? positions[tok] : -1;
+  [[maybe_unused]] const float row_mul =
+      SHAPED ? scale_log2e * (1.0f / ZA_LOG2E) * query_temperature(ex, pos_row) : 0.f;
   const int lo = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
   const int hi = pos_last;
   int range_lo = z * keys_per_split;
@@ -997,7 +1030,9 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
         const int kp = tile0 + (jb >> 1) * 32 + grp * 8 + (jb & 1) * 4 + i;
         bool valid = kp <= pos_row && kp >= lo && kp <= range_hi;
         if (window > 0 && kp <= pos_row - window) valid = false;
-        const float v = valid ? s[jb][i] * scale_log2e : -INFINITY;
+        const float v = valid ? (SHAPED ? shaped_score_log2(ex, s[jb][i], row_mul)
+                                        : s[jb][i] * scale_log2e)
+                              : -INFINITY;
         s[jb][i] = v;
         tmax = fmaxf(tmax, v);
       }
@@ -1067,6 +1102,8 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
       wgt[w] = mg_m[w][r16] > -INFINITY ? ldexpf(1.0f, (int)(mg_m[w][r16] - mu)) : 0.f;
       total += mg_l[w][r16] * wgt[w];
     }
+    if (SHAPED && ex.sink && nsplit == 1 && mx > -INFINITY)
+      total += exp2f(ex.sink[head] * ZA_LOG2E - mu);
     const size_t orow = (size_t)tok * nh + head;
 #pragma unroll
     for (int db = 0; db < DBLK; ++db)
@@ -1254,16 +1291,16 @@ static int paged_attention_any(const void* q, void* out, const void* kv, const i
   return za_head_gate(out, gate, dtype, gate_stride, gate_col, n_tokens, nh, dv, out_scale, stream);
 }
 
-template <int D, int KT>
+template <int D, int KT, bool SHAPED>
 static int launch_attention_mfma(const void* q, void* out, const void* kv, const int* block_table,
                                  int bt_stride, const int* positions, const int* wi_seq,
                                  const int* wi_row0, const int* wi_count, int n_items,
                                  int n_tokens, float* part_acc, float* part_ml, int nh, int nkv,
                                  int page_size, float scale, int window, int keys_per_split,
-                                 int nsplit, hipStream_t stream) {
+                                 int nsplit, ScoreExtras ex, hipStream_t stream) {
   constexpr int NW = 8, NS = AM_ROWS / (NW * 16);
   const size_t shmem = ((size_t)2 * KT * (D + 8) + (size_t)2 * D * (KT + 8)) * sizeof(bf16_t);
-  auto kernel = paged_attention_mfma_kernel<D, NW, NS, KT>;
+  auto kernel = paged_attention_mfma_kernel<D, NW, NS, KT, SHAPED>;
   static bool allowed = false;
   if (!allowed) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel,
@@ -1278,12 +1315,12 @@ static int launch_attention_mfma(const void* q, void* out, const void* kv, const
   hipLaunchKernelGGL(kernel, grid, block, shmem, stream, (const bf16_t*)q, (bf16_t*)out,
                      (const bf16_t*)kv, block_table, bt_stride, positions, wi_seq, wi_row0,
                      wi_count, n_items, part_acc, part_ml, nh, nkv, page_size,
-                     scale * 1.44269504088896341f, window, keys_per_split, nsplit);
+                     scale * 1.44269504088896341f, window, keys_per_split, nsplit, ex);
   int rc = za_launch_status();
   if (rc != 0 || nsplit == 1) return rc;
   dim3 cgrid((unsigned)((size_t)n_tokens * nh)), cblock(64);
   hipLaunchKernelGGL((attention_combine_kernel<bf16_t>), cgrid, cblock, 0, stream, part_acc,
-                     part_ml, (bf16_t*)out, D, nsplit, 1, nullptr, 1);
+                     part_ml, (bf16_t*)out, D, nsplit, 1, SHAPED ? ex.sink : nullptr, nh);
   return za_launch_status();
 }
 
@@ -1291,14 +1328,12 @@ static int launch_attention_mfma(const void* q, void* out, const void* kv, const
 // multiples of 4, a positive scale, work items of at most 128 / (nh / nkv) query
 // tokens; contexts optionally cut as in za_paged_attention (partial results merged by
 // the same combine kernel).  Returns ZA_ERR_UNSUPPORTED otherwise.
-extern "C" int za_paged_attention_mfma(const void* q, void* out, const void* kv,
-                                       const int* block_table, int bt_stride,
-                                       const int* positions, const int* wi_seq,
-                                       const int* wi_row0, const int* wi_count, int n_items,
-                                       int n_tokens, float* part_acc, float* part_ml, int nh,
-                                       int nkv, int d, int page_size, float scale, int window,
-                                       int keys_per_split, int nsplit, int tile_keys,
-                                       hipStream_t stream) {
+static int attention_mfma_any(const void* q, void* out, const void* kv, const int* block_table,
+                              int bt_stride, const int* positions, const int* wi_seq,
+                              const int* wi_row0, const int* wi_count, int n_items, int n_tokens,
+                              float* part_acc, float* part_ml, int nh, int nkv, int d,
+                              int page_size, float scale, int window, int keys_per_split,
+                              int nsplit, int tile_keys, ScoreExtras ex, hipStream_t stream) {
   if (n_items == 0 || n_tokens == 0) return 0;
   if (nsplit < 1 || nsplit > 65535 ||
       (nsplit > 1 && (!part_acc || !part_ml || keys_per_split <= 0 || keys_per_split % 64 != 0)))
@@ -1315,48 +1350,88 @@ extern "C" int za_paged_attention_mfma(const void* q, void* out, const void* kv,
     return ZA_ERR_UNSUPPORTED;
 #define ZA_AM_ARGS                                                                             \
   q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0, wi_count, n_items, n_tokens, \
-      part_acc, part_ml, nh, nkv, page_size, scale, window, keys_per_split, nsplit, stream
+      part_acc, part_ml, nh, nkv, page_size, scale, window, keys_per_split, nsplit, ex, stream
   // tiles of 128 keys spread a tile's fixed work (running maximum, addresses) over twice
   // the scores: for long contexts; head size 128 keeps tiles of 64 (LDS)
-  if (d == 64) return tile_keys == 128 ? launch_attention_mfma<64, 128>(ZA_AM_ARGS)
-                                       : launch_attention_mfma<64, 64>(ZA_AM_ARGS);
-  return launch_attention_mfma<128, 64>(ZA_AM_ARGS);
+  if (ex.softcap > 0.f || ex.sink || ex.qt_every > 0) {
+    if (d == 64) return tile_keys == 128 ? launch_attention_mfma<64, 128, true>(ZA_AM_ARGS)
+                                         : launch_attention_mfma<64, 64, true>(ZA_AM_ARGS);
+    return launch_attention_mfma<128, 64, true>(ZA_AM_ARGS);
+  }
+  if (d == 64) return tile_keys == 128 ? launch_attention_mfma<64, 128, false>(ZA_AM_ARGS)
+                                       : launch_attention_mfma<64, 64, false>(ZA_AM_ARGS);
+  return launch_attention_mfma<128, 64, false>(ZA_AM_ARGS);
 #undef ZA_AM_ARGS
 }
 
-template <bool ROPE>
+extern "C" int za_paged_attention_mfma(const void* q, void* out, const void* kv,
+                                       const int* block_table, int bt_stride,
+                                       const int* positions, const int* wi_seq,
+                                       const int* wi_row0, const int* wi_count, int n_items,
+                                       int n_tokens, float* part_acc, float* part_ml, int nh,
+                                       int nkv, int d, int page_size, float scale, int window,
+                                       int keys_per_split, int nsplit, int tile_keys,
+                                       hipStream_t stream) {
+  return attention_mfma_any(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0,
+                            wi_count, n_items, n_tokens, part_acc, part_ml, nh, nkv, d, page_size,
+                            scale, window, keys_per_split, nsplit, tile_keys,
+                            ScoreExtras{0.f, nullptr, 0.f, 0}, stream);
+}
+
+// The same with what `ScoreExtras` describes.
+extern "C" int za_paged_attention_mfma_shaped(const void* q, void* out, const void* kv,
+                                              const int* block_table, int bt_stride,
+                                              const int* positions, const int* wi_seq,
+                                              const int* wi_row0, const int* wi_count,
+                                              int n_items, int n_tokens, float* part_acc,
+                                              float* part_ml, int nh, int nkv, int d,
+                                              int page_size, float scale, int window,
+                                              int keys_per_split, int nsplit, int tile_keys,
+                                              float softcap, const float* sink, float qt_coef,
+                                              int qt_every, hipStream_t stream) {
+  if (softcap < 0.f || qt_every < 0) return ZA_ERR_ARG;
+  return attention_mfma_any(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0,
+                            wi_count, n_items, n_tokens, part_acc, part_ml, nh, nkv, d, page_size,
+                            scale, window, keys_per_split, nsplit, tile_keys,
+                            ScoreExtras{softcap, sink, qt_coef, qt_every}, stream);
+}
+
+template <bool ROPE, bool SHAPED = false>
 static int launch_decode_mfma(const void* q, void* out, const void* kv, const int* block_table,
                               int bt_stride, const int* positions, const int* wi_seq,
                               const int* wi_row0, const int* wi_count, int n_items, int n_tokens,
                               float* part_acc, float* part_ml, int nh, int nkv, int d,
                               int page_size, float scale, int window, int keys_per_split,
                               int nsplit, const DecodeRope& rope, bool combine,
-                              hipStream_t stream) {
+                              hipStream_t stream, ScoreExtras ex = ScoreExtras{0.f, nullptr, 0.f, 0}) {
   dim3 grid(n_items, nkv, nsplit), block(256);
   // Few workgroups (a small batch): eight waves each, so that a compute unit that
   // gets one workgroup still has eight waves' loads in flight.
   const long long workgroups = (long long)n_items * nkv * nsplit;
   if (d == 64 && workgroups <= ZA_DECODE_WIDE_BELOW) {
-    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<64, 8, ROPE>), grid, dim3(512), 0, stream,
+    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<64, 8, ROPE, SHAPED>), grid, dim3(512), 0, stream,
                        (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
                        positions, wi_seq, wi_row0, wi_count, part_acc, part_ml, nh, nkv,
-                       page_size, scale * 1.44269504088896341f, window, keys_per_split, nsplit, rope);
+                       page_size, scale * 1.44269504088896341f, window, keys_per_split, nsplit, rope,
+                       ex);
   } else if (d == 64) {
-    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<64, 4, ROPE>), grid, block, 0, stream,
+    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<64, 4, ROPE, SHAPED>), grid, block, 0, stream,
                        (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
                        positions, wi_seq, wi_row0, wi_count, part_acc, part_ml, nh, nkv,
-                       page_size, scale * 1.44269504088896341f, window, keys_per_split, nsplit, rope);
+                       page_size, scale * 1.44269504088896341f, window, keys_per_split, nsplit, rope,
+                       ex);
   } else {
-    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<128, 4, ROPE>), grid, block, 0, stream,
+    hipLaunchKernelGGL((paged_attention_decode_mfma_kernel<128, 4, ROPE, SHAPED>), grid, block, 0, stream,
                        (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kv, block_table, bt_stride,
                        positions, wi_seq, wi_row0, wi_count, part_acc, part_ml, nh, nkv,
-                       page_size, scale * 1.44269504088896341f, window, keys_per_split, nsplit, rope);
+                       page_size, scale * 1.44269504088896341f, window, keys_per_split, nsplit, rope,
+                       ex);
   }
   int rc = za_launch_status();
   if (rc != 0 || nsplit == 1 || !combine) return rc;
   dim3 cgrid((unsigned)((size_t)n_tokens * nh)), cblock(64);
   hipLaunchKernelGGL((attention_combine_kernel<bf16_t>), cgrid, cblock, 0, stream, part_acc,
-                     part_ml, (bf16_t*)out, d, nsplit, 1, nullptr, 1);
+                     part_ml, (bf16_t*)out, d, nsplit, 1, SHAPED ? ex.sink : nullptr, nh);
   return za_launch_status();
 }
 
@@ -1376,15 +1451,12 @@ extern "C" int za_attention_combine(const float* part_acc, const float* part_ml,
 // multiples of 4, work items of at most 16 / (nh / nkv) query tokens, contexts
 // optionally cut as in
 // za_paged_attention (the partial results are merged by the same combine kernel).
-extern "C" int za_paged_attention_decode_mfma(const void* q, void* out, const void* kv,
-                                              const int* block_table, int bt_stride,
-                                              const int* positions, const int* wi_seq,
-                                              const int* wi_row0, const int* wi_count,
-                                              int n_items, int n_tokens, float* part_acc,
-                                              float* part_ml, int nh, int nkv, int d,
-                                              int page_size, float scale, int window,
-                                              int keys_per_split, int nsplit,
-                                              hipStream_t stream) {
+static int decode_mfma_any(const void* q, void* out, const void* kv, const int* block_table,
+                           int bt_stride, const int* positions, const int* wi_seq,
+                           const int* wi_row0, const int* wi_count, int n_items, int n_tokens,
+                           float* part_acc, float* part_ml, int nh, int nkv, int d, int page_size,
+                           float scale, int window, int keys_per_split, int nsplit, ScoreExtras ex,
+                           hipStream_t stream) {
   if (n_items == 0 || n_tokens == 0) return 0;
   if (n_items < 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || page_size <= 0 || bt_stride <= 0 ||
       nsplit < 1 || !q || !out || !kv || !block_table || !positions)
@@ -1397,10 +1469,43 @@ extern "C" int za_paged_attention_decode_mfma(const void* q, void* out, const vo
   if (nsplit > 1 && (!part_acc || !part_ml || keys_per_split <= 0 || keys_per_split % 64 != 0))
     return ZA_ERR_ARG;
   const DecodeRope none = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.f, 0};
+  if (ex.softcap > 0.f || ex.sink || ex.qt_every > 0)
+    return launch_decode_mfma<false, true>(q, out, kv, block_table, bt_stride, positions, wi_seq,
+                                           wi_row0, wi_count, n_items, n_tokens, part_acc, part_ml,
+                                           nh, nkv, d, page_size, scale, window, keys_per_split,
+                                           nsplit, none, true, stream, ex);
   return launch_decode_mfma<false>(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0,
                                    wi_count, n_items, n_tokens, part_acc, part_ml, nh, nkv, d,
                                    page_size, scale, window, keys_per_split, nsplit, none, true,
                                    stream);
+}
+
+extern "C" int za_paged_attention_decode_mfma(const void* q, void* out, const void* kv,
+                                              const int* block_table, int bt_stride,
+                                              const int* positions, const int* wi_seq,
+                                              const int* wi_row0, const int* wi_count,
+                                              int n_items, int n_tokens, float* part_acc,
+                                              float* part_ml, int nh, int nkv, int d,
+                                              int page_size, float scale, int window,
+                                              int keys_per_split, int nsplit,
+                                              hipStream_t stream) {
+  return decode_mfma_any(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0, wi_count,
+                         n_items, n_tokens, part_acc, part_ml, nh, nkv, d, page_size, scale,
+                         window, keys_per_split, nsplit, ScoreExtras{0.f, nullptr, 0.f, 0}, stream);
+}
+
+// The same with what `ScoreExtras` describes.
+extern "C" int za_paged_attention_decode_mfma_shaped(
+    const void* q, void* out, const void* kv, const int* block_table, int bt_stride,
+    const int* positions, const int* wi_seq, const int* wi_row0, const int* wi_count, int n_items,
+    int n_tokens, float* part_acc, float* part_ml, int nh, int nkv, int d, int page_size,
+    float scale, int window, int keys_per_split, int nsplit, float softcap, const float* sink,
+    float qt_coef, int qt_every, hipStream_t stream) {
+  if (softcap < 0.f || qt_every < 0) return ZA_ERR_ARG;
+  return decode_mfma_any(q, out, kv, block_table, bt_stride, positions, wi_seq, wi_row0, wi_count,
+                         n_items, n_tokens, part_acc, part_ml, nh, nkv, d, page_size, scale,
+                         window, keys_per_split, nsplit,
+                         ScoreExtras{softcap, sink, qt_coef, qt_every}, stream);
 }
 
 // The same for a step in which every request brings one token, with the token's part of

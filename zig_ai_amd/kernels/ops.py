@@ -127,6 +127,14 @@ _SIGNATURES = {
                                                  c_int, c_void_p, c_void_p, c_int, c_int, c_int,
                                                  c_int, c_int, c_int, c_float, c_int, c_int, c_int,
                                                  c_float, c_void_p, c_float, c_int, c_void_p],
+    ("attention", "za_paged_attention_mfma_shaped"): [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+        c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
+        c_int, c_float, c_void_p, c_float, c_int, c_void_p],
+    ("attention", "za_paged_attention_decode_mfma_shaped"): [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+        c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
+        c_float, c_void_p, c_float, c_int, c_void_p],
     ("experts", "za_expert_lists"): [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
                                      c_void_p, c_void_p],
     ("experts", "za_grouped_gemm"): [c_void_p, c_int, c_longlong, c_void_p, c_int, c_void_p,
@@ -1093,7 +1101,8 @@ def paged_attention_mfma(q: torch.Tensor, kv_cache: torch.Tensor, block_table: t
                          positions: torch.Tensor, item_seq: torch.Tensor,
                          item_row0: torch.Tensor, item_count: torch.Tensor, n_items: int,
                          scale: float, window: int = 0, keys_per_split: int = 0,
-                         nsplit: int = 1, tile_keys: int = 64) -> torch.Tensor:
+                         nsplit: int = 1, tile_keys: int = 64,
+                         shape: Optional[ScoreShape] = None) -> torch.Tensor:
     """The same attention on the matrix cores (bfloat16, head_dim 64 or 128, at most
     16 query heads per key/value head, a page size that is a multiple of 4, a
     positive scale).  Work items hold at most
@@ -1130,11 +1139,18 @@ def paged_attention_mfma(q: torch.Tensor, kv_cache: torch.Tensor, block_table: t
             raise KernelError("keys_per_split must be a positive multiple of 64")
         part_acc = torch.empty((T, nh, nsplit, d), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T, nh, nsplit, 2), dtype=torch.float32, device=q.device)
-    rc = _fn("attention", "za_paged_attention_mfma")(
-        _ptr(q), _ptr(out), _ptr(kv_cache), _ptr(block_table), block_table.shape[1],
-        _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
-        _ptr(part_acc), _ptr(part_ml), nh, nkv, d, page_size, float(scale), int(window),
-        int(keys_per_split), int(nsplit), int(tile_keys), _stream())
+    if shape:
+        rc = _fn("attention", "za_paged_attention_mfma_shaped")(
+            _ptr(q), _ptr(out), _ptr(kv_cache), _ptr(block_table), block_table.shape[1],
+            _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
+            _ptr(part_acc), _ptr(part_ml), nh, nkv, d, page_size, float(scale), int(window),
+            int(keys_per_split), int(nsplit), int(tile_keys), *shape.args(nh), _stream())
+    else:
+        rc = _fn("attention", "za_paged_attention_mfma")(
+            _ptr(q), _ptr(out), _ptr(kv_cache), _ptr(block_table), block_table.shape[1],
+            _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
+            _ptr(part_acc), _ptr(part_ml), nh, nkv, d, page_size, float(scale), int(window),
+            int(keys_per_split), int(nsplit), int(tile_keys), _stream())
     _check(rc, "paged_attention_mfma")
     _note("attention", kernel="mfma", rows=T, dtype=q.dtype, nsplit=int(nsplit))
     return out
@@ -1149,7 +1165,7 @@ def paged_attention_decode_mfma(q: torch.Tensor, kv_cache: torch.Tensor,
                                 item_row0: Optional[torch.Tensor],
                                 item_count: Optional[torch.Tensor], n_items: int, scale: float,
                                 window: int = 0, keys_per_split: int = 0,
-                                nsplit: int = 1) -> torch.Tensor:
+                                nsplit: int = 1, shape: Optional[ScoreShape] = None) -> torch.Tensor:
     """The matrix-core kernel for decoding: work items of at most
     ``ATTENTION_MFMA_DECODE_ROWS // (heads // kv_heads)`` query tokens, long contexts
     optionally cut into ``nsplit`` ranges of ``keys_per_split`` keys.  With
@@ -1186,11 +1202,18 @@ def paged_attention_decode_mfma(q: torch.Tensor, kv_cache: torch.Tensor,
             raise KernelError("keys_per_split must be a positive multiple of 64")
         part_acc = torch.empty((T, nh, nsplit, d), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((T, nh, nsplit, 2), dtype=torch.float32, device=q.device)
-    rc = _fn("attention", "za_paged_attention_decode_mfma")(
-        _ptr(q), _ptr(out), _ptr(kv_cache), _ptr(block_table), block_table.shape[1],
-        _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
-        _ptr(part_acc), _ptr(part_ml), nh, nkv, d, page_size, float(scale), int(window),
-        int(keys_per_split), int(nsplit), _stream())
+    if shape:
+        rc = _fn("attention", "za_paged_attention_decode_mfma_shaped")(
+            _ptr(q), _ptr(out), _ptr(kv_cache), _ptr(block_table), block_table.shape[1],
+            _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
+            _ptr(part_acc), _ptr(part_ml), nh, nkv, d, page_size, float(scale), int(window),
+            int(keys_per_split), int(nsplit), *shape.args(nh), _stream())
+    else:
+        rc = _fn("attention", "za_paged_attention_decode_mfma")(
+            _ptr(q), _ptr(out), _ptr(kv_cache), _ptr(block_table), block_table.shape[1],
+            _ptr(positions), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), n_items, T,
+            _ptr(part_acc), _ptr(part_ml), nh, nkv, d, page_size, float(scale), int(window),
+            int(keys_per_split), int(nsplit), _stream())
     _check(rc, "paged_attention_decode_mfma")
     _note("attention", kernel="decode_mfma", rows=T, dtype=q.dtype, nsplit=int(nsplit))
     return out

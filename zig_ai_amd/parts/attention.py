@@ -172,6 +172,9 @@ class GroupedQueryAttention(Mixer):
         if self.wide:
             self.w_qkv = ops.projection_weight(pad_rows(self.w_qkv))
             self.w_out = ops.projection_weight(self.w_out)
+        elif self.shared_values or self.shape:
+            self.w_qkv = ops.projection_weight(self.w_qkv)
+            self.w_out = ops.projection_weight(self.w_out)
         self.b_qkv = self.b_out = None
         if params.get("bias"):
             b = torch.cat([tensors["q_proj.bias"], tensors["k_proj.bias"], tensors["v_proj.bias"]])
@@ -191,7 +194,7 @@ class GroupedQueryAttention(Mixer):
         if self.wide and self.position is not None and not self.fused_rotation:
             raise ValueError("an attention with value_dim or gate takes a rotary position "
                              "encoding or none")
-        self.mfma = self.mfma and self.value_dim == self.head_dim and not self.shape
+        self.mfma = self.mfma and self.value_dim == self.head_dim
         if self.shape and self.wide:
             raise ValueError("a cap, a sink or a query temperature go with values of the keys' "
                              "width and no gate")
@@ -266,7 +269,8 @@ class GroupedQueryAttention(Mixer):
             # faster from 512 tokens to 32,768); head size 128 keeps tiles of 64 (LDS)
             o = ops.paged_attention_mfma(q, cache.kv, step.block_tables[cache.group],
                                          step.positions, *items, self.scale, self.window,
-                                         keys, nsplit, tile_keys=128 if d == 64 else 64)
+                                         keys, nsplit, tile_keys=128 if d == 64 else 64,
+                                         shape=self.shape)
         elif mfma:
             # single tokens only: the matrix-core kernel whose waves split the keys
             # (every request brings one token: row i is request i, no work-item arrays)
@@ -275,7 +279,8 @@ class GroupedQueryAttention(Mixer):
             keys, nsplit = plan_split(n_items, nkv, step.max_keys)
             o = ops.paged_attention_decode_mfma(q, cache.kv, step.block_tables[cache.group],
                                                 step.positions, item_seq, item_row0, item_count,
-                                                n_items, self.scale, self.window, keys, nsplit)
+                                                n_items, self.scale, self.window, keys, nsplit,
+                                                shape=self.shape)
         else:
             item_seq, item_row0, item_count, n_items = step.attention_items(self.rows_per_item)
             keys, nsplit = plan_split(n_items, nkv, step.max_keys)
