@@ -134,8 +134,8 @@ class GroupedQueryAttention(Mixer):
         if self.group > ops.ATTENTION_MAX_ROWS:
             raise ValueError(f"{self.group} query heads per key/value head exceed the attention "
                              f"kernel's limit of {ops.ATTENTION_MAX_ROWS}")
-        # (the kernels that take the cache as two planes read eight elements at a time)
-        multiple = 8 if self.wide else 16
+        # (the general kernels read eight elements at a time)
+        multiple = 8
         if self.head_dim % multiple or self.head_dim > 256:
             raise ValueError(f"head_dim {self.head_dim} must be a multiple of {multiple}, at most 256")
         # tokens per work item of the two attention kernels
