@@ -4,6 +4,7 @@
     python bench.py --shape 2.6b --prompt-len 6144        # another LFM2 shape, same measurement
     python bench.py --shape 350m --workload serve         # 64 requests through the scheduler
     python bench.py --workload compare                    # Rudilix beside LFM2 at equal sizes
+    python bench.py --workload compare --compare-design ranesun   # Ranesun beside Rudilix
 
 Default run: the layer sizes of the LFM2-1.2B shape (16 layers, hidden 2048, vocabulary 65,536)
 with random bfloat16 weights N(0, 0.02), a batch of 8 requests, each prefilled
@@ -31,7 +32,10 @@ The model is ``DecoderModel.from_random(cfg, seed=0)``: the tensors that
 rule, state-space and delta layers) and an LFM2 model of the same width, depth,
 feed-forward width and vocabulary, attention where the other has it, both with random
 weights: a 2,048-token prefill and decode steps of a batch of 8 at that context, per
-width (``--compare-widths``), as one JSON line.
+width (``--compare-widths``), as one JSON line.  ``--compare-design ranesun``: a Ranesun model
+(retention and sink attention layers in turn, dense and table-routed feed-forwards in turn,
+the first half of the layers as a looped span) beside a Rudilix model of the same width,
+depth and vocabulary, the closest design the engine has (recurrent and attention layers).
 """
 
 import argparse
@@ -155,8 +159,34 @@ def rudilix_shape(width, layers, vocab):
             "norm": {"eps": 1e-5}, "layers": out, "max_position_embeddings": 128000}
 
 
-def compare(widths, layers, batch, prompt_len, steps, warmup) -> dict:
-    """Prefill and decode throughput of Rudilix and of LFM2 at equal sizes."""
+def ranesun_shape(width, layers, vocab):
+    """Layer sizes in the manner of a real model of this design: retention layers (keys of
+    64, values of 128, decays spread from 1 - 2^-5 to 1 - 2^-12) and attention layers (heads
+    of 64 in groups of eight a key head, whose values are the keys) in turn; feed-forwards
+    in turn dense (four times the width) and eight experts of twice the width of which a
+    token uses two; the first half of the layers a looped span that runs once."""
+    heads = width // 128
+    retention = {"heads": heads, "dim": 64, "vdim": 128,
+                 "decay": [1.0 - 2.0 ** -(5 + 7 * h / max(1, heads - 1)) for h in range(heads)],
+                 "rot": {"dims": 64, "base": 1e6}}
+    q_heads = width // 64
+    attention = {"heads": q_heads, "kv_heads": max(1, q_heads // 8), "dim": 64, "vdim": 64,
+                 "scale": 0.125, "softcap": 30.0, "q_temp": {"coef": 0.5, "every": 1024}}
+    dense = {"kind": "dense", "ff": 4 * width}
+    moe = {"kind": "moe", "expert": {"ff": 2 * width}, "router": {"experts": 8, "top": 2}}
+    out = []
+    for i in range(layers):
+        kind = "retention" if i % 2 == 0 else "attention"
+        out.append({"type": kind, "mixer": retention if kind == "retention" else attention,
+                    "mlp": dense if (i // 2) % 2 == 0 else moe})
+    return {"architecture": "Ranesun", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+            "logit_scale": 1.0, "loop": {"start": 0, "stop": max(1, layers // 2), "times": 1},
+            "layers": out, "max_position_embeddings": 128000}
+
+
+def compare(widths, layers, batch, prompt_len, steps, warmup, design="rudilix", only=None) -> dict:
+    """Prefill and decode throughput of Rudilix and of LFM2 at equal sizes, or
+    (``design="ranesun"``) of Ranesun and of Rudilix."""
     import torch
     from zig_ai_amd.engine import DecoderModel, ModelRunner, StepEntry
     from zig_ai_amd.kernels import ops
@@ -245,6 +275,13 @@ def compare(widths, layers, batch, prompt_len, steps, warmup) -> dict:
 
     result = {"workload": "compare", "dtype": "bf16", "data": "synthetic", "layers": layers,
               "batch": batch, "prompt_len": prompt_len, "steps": steps, "warmup": warmup, "widths": {}}
+    if design == "ranesun":
+        for width in widths:
+            pair = {"ranesun": ranesun_shape, "rudilix": rudilix_shape}
+            result["widths"][str(width)] = {name: measure(shape(width, layers, vocab))
+                                            for name, shape in pair.items()
+                                            if only in (None, name)}
+        return result
     for width in widths:
         new = rudilix_shape(width, layers, vocab)
         attention_at = tuple(i for i, l in enumerate(new["layers"]) if l["type"] == "parallel")
@@ -300,6 +337,10 @@ def main() -> int:
     ap.add_argument("--compare-widths", default="1024,2048",
                     help="--workload compare: the widths, with commas between them")
     ap.add_argument("--compare-layers", type=int, default=8, help="--workload compare: layers")
+    ap.add_argument("--compare-design", choices=["rudilix", "ranesun"], default="rudilix",
+                    help="--workload compare: rudilix (beside LFM2) or ranesun (beside Rudilix)")
+    ap.add_argument("--compare-only", default=None,
+                    help="--workload compare: measure this model of the pair alone (for a profiler)")
     ap.add_argument("--workload", choices=["steps", "serve", "compare"], default="steps",
                     help="steps: decode steps and one prefill (the default run); serve: 64 "
                          "requests with prompts of 128-2048 tokens and 256 new tokens each "
@@ -336,7 +377,8 @@ def main() -> int:
     if args.workload == "compare":
         print(json.dumps(compare([int(w) for w in args.compare_widths.split(",")],
                                  args.compare_layers, args.batch, args.prompt_len, args.steps,
-                                 args.warmup)), flush=True)
+                                 args.warmup, args.compare_design, args.compare_only)),
+              flush=True)
         return 0
     if args.workload == "serve":
         print(json.dumps(serve(cfg, args.shape.upper(), args.requests, args.new_tokens,

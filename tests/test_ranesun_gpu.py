@@ -544,7 +544,9 @@ def test_retention_kernels(H, d, dv, rot):
                                                 (3, 8, 2, 320, 96, torch.bfloat16),
                                                 (130, 3, 3, 40, 72, torch.bfloat16),
                                                 (9, 1, 1, 24, 8, torch.float32),
-                                                (600, 64, 4, 64, 40, torch.bfloat16)])
+                                                (600, 64, 4, 64, 40, torch.bfloat16),
+                                                (1200, 4, 2, 72, 136, torch.bfloat16),
+                                                (700, 2, 1, 256, 200, torch.bfloat16)])
 def test_expert_kernels(T, E, top, K, N, dtype):
     from zig_ai_amd.kernels import ops
     dev = torch.device("cuda")

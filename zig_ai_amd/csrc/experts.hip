@@ -25,7 +25,11 @@
 //      bfloat16: matrix cores (v_mfma_f32_16x16x32_bf16), operands straight from memory
 //      into the fragments; TM = 64 (four waves, 16 rows x 64 columns each) for steps with
 //      prompt portions, TM = 16 (four waves, 16 columns each) for decode batches, where an
-//      expert has a token or two and the weights are all that moves.
+//      expert has a token or two and the weights are all that moves; for steps of many
+//      tokens an expert (128 and more on average) tiles of 128 x 128 through LDS, a step of
+//      64 of K at a time with the next step's pieces on their way into registers, four
+//      waves of 64 x 64 each: every element of either operand is then read from memory
+//      once a tile and used 128 times.
 //      32-bit: LDS-tiled FMA, 64 x 64 tiles (no matrix-core rounding mode).
 #include "common.h"
 
@@ -181,6 +185,106 @@ grouped_gemm_bf16_kernel(GroupedArgs g) {
   }
 }
 
+// Tiles of 128 assignments x 128 outputs through LDS, for experts with many rows.
+#define GG_BM 128
+#define GG_BN 128
+#define GG_BK 64
+#define GG_LD (GG_BK + 8)   // padded row, in elements: spreads rows over LDS banks
+
+template <typename TO>
+__global__ void __launch_bounds__(256)
+grouped_gemm_bf16_tiled_kernel(GroupedArgs g) {
+  __shared__ __attribute__((aligned(16))) bf16_t As[GG_BM * GG_LD];
+  __shared__ __attribute__((aligned(16))) bf16_t Ws[GG_BN * GG_LD];
+  int e, tile, count;
+  if (!find_tile<GG_BM>(g.counts, g.E, blockIdx.x, &e, &tile, &count)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int n0 = blockIdx.y * GG_BN;
+  const int* mine = g.lists + (size_t)e * g.A;
+  const int K = g.K, N = g.N;
+  const bf16_t* wbase = (const bf16_t*)g.W + (size_t)e * N * K;
+
+  f32x4_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+  // a thread moves 4 + 4 pieces of 8 elements a step: rows lrow + 32 i, elements lcol .. + 7
+  const int lrow = tid >> 3, lcol = (tid & 7) * 8;
+  const bf16_t* arow[4];
+  const bf16_t* wrow[4];
+  bool a_ok[4], w_ok[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = tile * GG_BM + lrow + 32 * i, n = n0 + lrow + 32 * i;
+    a_ok[i] = r < count;
+    w_ok[i] = n < N;
+    arow[i] = (const bf16_t*)g.src + (size_t)(a_ok[i] ? mine[r] / g.src_div : 0) * K;
+    wrow[i] = wbase + (size_t)(w_ok[i] ? n : 0) * K;
+  }
+  bf16x8_t ra[4], rw[4];
+  const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  auto fetch = [&](int k0) {
+    const int k = k0 + lcol;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      ra[i] = (a_ok[i] && k < K) ? *reinterpret_cast<const bf16x8_t*>(arow[i] + k) : zero8;
+      rw[i] = (w_ok[i] && k < K) ? *reinterpret_cast<const bf16x8_t*>(wrow[i] + k) : zero8;
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      *reinterpret_cast<bf16x8_t*>(As + (lrow + 32 * i) * GG_LD + lcol) = ra[i];
+      *reinterpret_cast<bf16x8_t*>(Ws + (lrow + 32 * i) * GG_LD + lcol) = rw[i];
+    }
+  };
+  fetch(0);
+  stash();
+  __syncthreads();
+  const int r16 = lane & 15, kq = (lane >> 4) * 8;
+  for (int k0 = 0; k0 < K; k0 += GG_BK) {
+    const bool more = k0 + GG_BK < K;
+    if (more) fetch(k0 + GG_BK);
+#pragma unroll
+    for (int ks = 0; ks < GG_BK; ks += 32) {
+      bf16x8_t fa[4], fw[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        fa[i] = *reinterpret_cast<const bf16x8_t*>(As + (wm * 64 + i * 16 + r16) * GG_LD + ks + kq);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        fw[j] = *reinterpret_cast<const bf16x8_t*>(Ws + (wn * 64 + j * 16 + r16) * GG_LD + ks + kq);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+    if (more) {
+      stash();
+      __syncthreads();
+    }
+  }
+  TO* out = (TO*)g.out;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int row = tile * GG_BM + wm * 64 + i * 16 + (lane >> 4) * 4 + r;
+      if (row >= count) continue;
+      const size_t d = dst_row(g, mine[row]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int n = n0 + wn * 64 + j * 16 + r16;
+        if (n < N) out[d * N + n] = from_f32<TO>(expert_act(acc[i][j][r], g.act) * g.out_scale);
+      }
+    }
+}
+
 // 32-bit weights (src of either type): 64 x 64 tiles through LDS, plain FMA.
 template <typename TA, typename TO>
 __global__ void __launch_bounds__(256)
@@ -262,6 +366,17 @@ extern "C" int za_grouped_gemm(const void* src, int src_dtype, long long src_row
   const unsigned ntiles = (unsigned)((N + 63) / 64);
   if (w_dtype == 1) {
     if (src_dtype != 1 || K % 8 != 0) return ZA_ERR_UNSUPPORTED;
+    if (A >= 128LL * experts) {
+      // many rows an expert: tiles of 128 x 128 through LDS
+      dim3 grid((unsigned)((A + GG_BM - 1) / GG_BM + experts), (unsigned)((N + GG_BN - 1) / GG_BN));
+      if (out_dtype == 0)
+        hipLaunchKernelGGL((grouped_gemm_bf16_tiled_kernel<float>), grid, dim3(256), 0, stream, g);
+      else if (out_dtype == 1)
+        hipLaunchKernelGGL((grouped_gemm_bf16_tiled_kernel<bf16_t>), grid, dim3(256), 0, stream, g);
+      else
+        return ZA_ERR_UNSUPPORTED;
+      return za_launch_status();
+    }
     // a decode batch (an expert has a token or two): tiles of 16 rows
     const bool small = A <= 4LL * experts || A <= 64;
     const int TM = small ? 16 : 64;
