@@ -60,13 +60,24 @@ __device__ __forceinline__ float capped_score(const ScoreExtras& ex, float s) {
 // `dot * row_mul` (row_mul: scale times the row's temperature), capped, times log2(e).
 // tanh(x) = 1 - 2 / (exp(2x) + 1) with the hardware's exp2 and reciprocal: an absolute
 // error of some 1e-7 in tanh, far below what rounding the probabilities to bfloat16 does.
-__device__ __forceinline__ float shaped_score_log2(const ScoreExtras& ex, float dot, float row_mul) {
-  float s = dot * row_mul;
+// What does not depend on the key is folded into two numbers a row beforehand
+// (`shaped_row`): with a cap  a = row_mul * 2 log2(e) / cap,  b = cap * log2(e)  and the
+// score is  b - 2 b / (exp2(dot * a) + 1);  without one  a = row_mul * log2(e)  and the score
+// is  dot * a.  Three vector operations and the two transcendental ones a score.
+struct ShapedRow { float a, b; };
+
+__device__ __forceinline__ ShapedRow shaped_row(const ScoreExtras& ex, float row_mul) {
+  if (ex.softcap > 0.f)
+    return ShapedRow{row_mul * (2.0f * ZA_LOG2E / ex.softcap), ex.softcap * ZA_LOG2E};
+  return ShapedRow{row_mul * ZA_LOG2E, 0.f};
+}
+
+__device__ __forceinline__ float shaped_score_log2(const ScoreExtras& ex, float dot, ShapedRow r) {
   if (ex.softcap > 0.f) {
-    const float e = __builtin_amdgcn_exp2f(s * (2.0f * ZA_LOG2E / ex.softcap));
-    s = ex.softcap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f));
+    const float e = __builtin_amdgcn_exp2f(dot * r.a);
+    return fmaf(-2.0f * r.b, __builtin_amdgcn_rcpf(e + 1.0f), r.b);
   }
-  return s * ZA_LOG2E;
+  return dot * r.a;
 }
 
 #define AT_WAVES 4
@@ -421,7 +432,7 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
   int tok[NS], head[NS], pos_row[NS];
   bool row_valid[NS];
   bf16x8_t qf[NS][KSTEPS];
-  [[maybe_unused]] float row_mul[NS];
+  [[maybe_unused]] ShapedRow row_mul[NS];
   const float sl2 = SHAPED ? 1.0f : scale_log2e;   // shaped scores are on the base-2 scale already
 #pragma unroll
   for (int c = 0; c < NS; ++c) {
@@ -430,7 +441,8 @@ paged_attention_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ o
     tok[c] = row0 + (row_valid[c] ? rr / G : 0);
     head[c] = gkv * G + (row_valid[c] ? rr % G : 0);
     pos_row[c] = row_valid[c] ? positions[tok[c]] : -1;
-    if (SHAPED) row_mul[c] = scale_log2e * (1.0f / ZA_LOG2E) * query_temperature(ex, pos_row[c]);
+    if (SHAPED)
+      row_mul[c] = shaped_row(ex, scale_log2e * (1.0f / ZA_LOG2E) * query_temperature(ex, pos_row[c]));
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks)
       qf[c][ks] = row_valid[c] ? *reinterpret_cast<const bf16x8_t*>(
@@ -886,8 +898,8 @@ paged_attention_decode_mfma_kernel(const bf16_t* __restrict__ q, bf16_t* __restr
   const int pos_first = positions[row0];
   const int pos_last = positions[row0 + count - 1];
   const int pos_row = row_valid ? positions[tok] : -1;
-  [[maybe_unused]] const float row_mul =
-      SHAPED ? scale_log2e * (1.0f / ZA_LOG2E) * query_temperature(ex, pos_row) : 0.f;
+  [[maybe_unused]] const ShapedRow row_mul =
+      shaped_row(ex, SHAPED ? scale_log2e * (1.0f / ZA_LOG2E) * query_temperature(ex, pos_row) : 0.f);
   const int lo = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
   const int hi = pos_last;
   int range_lo = z * keys_per_split;
