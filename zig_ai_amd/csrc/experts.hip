@@ -152,11 +152,13 @@ grouped_gemm_bf16_kernel(GroupedArgs g) {
   for (int j = 0; j < NT; ++j) acc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  for (int k0 = 0; k0 < K; k0 += 64) {
-    // two steps of 32 a round: their loads are all requested before the first product
-    bf16x8_t fa[2], fw[2][NT];
+  // steps of 32 a round (two, or four where a wave has one column tile: a decode batch,
+  // which only streams weights): their loads are all requested before the first product
+  constexpr int U = NT == 1 ? 4 : 2;
+  for (int k0 = 0; k0 < K; k0 += 32 * U) {
+    bf16x8_t fa[U], fw[U][NT];
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
+    for (int s = 0; s < U; ++s) {
       const int k = k0 + s * 32 + kq * 8;
       const bool k_ok = k < K;           // K is a multiple of 8: a piece is inside or outside
       fa[s] = (row_ok && k_ok) ? *reinterpret_cast<const bf16x8_t*>(arow + k) : zero;
@@ -165,7 +167,7 @@ grouped_gemm_bf16_kernel(GroupedArgs g) {
         fw[s][j] = (col_ok[j] && k_ok) ? *reinterpret_cast<const bf16x8_t*>(wrow[j] + k) : zero;
     }
 #pragma unroll
-    for (int s = 0; s < 2; ++s)
+    for (int s = 0; s < U; ++s)
 #pragma unroll
       for (int j = 0; j < NT; ++j)
         acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[s], fw[s][j], acc[j], 0, 0, 0);
@@ -191,8 +193,12 @@ grouped_gemm_bf16_kernel(GroupedArgs g) {
 #define GG_BK 64
 #define GG_LD (GG_BK + 8)   // padded row, in elements: spreads rows over LDS banks
 
+#ifndef GG_MIN_WAVES
+#define GG_MIN_WAVES 2    // waves a SIMD the register budget is cut for
+#endif
+
 template <typename TO>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, GG_MIN_WAVES)
 grouped_gemm_bf16_tiled_kernel(GroupedArgs g) {
   __shared__ __attribute__((aligned(16))) bf16_t As[GG_BM * GG_LD];
   __shared__ __attribute__((aligned(16))) bf16_t Ws[GG_BN * GG_LD];

@@ -700,6 +700,51 @@ gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ gate,
   }
 }
 
+// The same for groups of at most 256 columns (a head's width): a wave a group, four
+// groups a workgroup, the group's values in registers, the sum over the wave's lanes
+// alone (no barrier).  grid: ceil(tokens * groups / 4).
+template <typename T>
+__global__ void __launch_bounds__(256)
+gated_group_norm_wave_kernel(const float* __restrict__ y, const T* __restrict__ gate,
+                             int gate_stride, int gate_col, const float* __restrict__ w, int wlen,
+                             T* __restrict__ out, int out_stride, int out_col, int width, int group,
+                             float eps, int silu_gate, int gate_first, float out_scale,
+                             long long n_groups_total) {
+  const int lane = threadIdx.x & 63;
+  const long long gi = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (gi >= n_groups_total) return;
+  const int per_token = width / group;
+  const size_t t = (size_t)(gi / per_token);
+  const int c0 = (int)(gi % per_token) * group;
+  const float* yr = y + t * width + c0;
+  const T* gr = gate + t * gate_stride + gate_col + c0;
+  T* o = out + t * out_stride + out_col + c0;
+  float v[4], act[4], wv[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int i = lane + 64 * k;
+    v[k] = i < group ? yr[i] : 0.f;
+    act[k] = i < group ? to_f32<T>(gr[i]) : 0.f;
+    wv[k] = i < group ? w[(c0 + i) % wlen] : 0.f;
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    act[k] = silu_gate ? silu_f(act[k]) : sigmoid_f(act[k]);
+    if (gate_first) v[k] *= act[k];
+    ss += v[k] * v[k];
+  }
+  ss = wave_sum(ss);
+  const float scale = 1.0f / sqrtf(ss / (float)group + eps);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int i = lane + 64 * k;
+    float r = v[k] * scale * wv[k];
+    if (!gate_first) r *= act[k];
+    if (i < group) o[i] = from_f32<T>(r * out_scale);
+  }
+}
+
 extern "C" int za_gated_group_norm(const float* y, const void* gate, int dtype, int gate_stride,
                                    int gate_col, const float* w, int wlen, void* out,
                                    int out_stride, int out_col, int n_tokens, int width, int group,
@@ -710,6 +755,21 @@ extern "C" int za_gated_group_norm(const float* y, const void* gate, int dtype, 
       wlen <= 0 || gate_col < 0 || gate_col + width > gate_stride || out_col < 0 ||
       out_col + width > out_stride)
     return ZA_ERR_ARG;
+  if (group <= 256 && dtype >= 0 && dtype <= 1) {
+    // small groups (a head each): a wave a group
+    const long long total = (long long)n_tokens * (width / group);
+    dim3 wgrid((unsigned)((total + 3) / 4)), wblock(256);
+    if (dtype == 0)
+      hipLaunchKernelGGL((gated_group_norm_wave_kernel<float>), wgrid, wblock, 0, stream, y,
+                         (const float*)gate, gate_stride, gate_col, w, wlen, (float*)out, out_stride,
+                         out_col, width, group, eps, silu_gate, gate_first, out_scale, total);
+    else
+      hipLaunchKernelGGL((gated_group_norm_wave_kernel<bf16_t>), wgrid, wblock, 0, stream, y,
+                         (const bf16_t*)gate, gate_stride, gate_col, w, wlen, (bf16_t*)out,
+                         out_stride, out_col, width, group, eps, silu_gate, gate_first, out_scale,
+                         total);
+    return za_launch_status();
+  }
   dim3 grid(n_tokens, width / group), block(group <= 64 ? 64 : (group <= 128 ? 128 : 256));
   if (dtype == 0)
     hipLaunchKernelGGL((gated_group_norm_kernel<float>), grid, block, 0, stream, y,
