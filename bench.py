@@ -168,10 +168,10 @@ def ranesun_shape(width, layers, vocab):
     heads = width // 128
     retention = {"heads": heads, "dim": 64, "vdim": 128,
                  "decay": [1.0 - 2.0 ** -(5 + 7 * h / max(1, heads - 1)) for h in range(heads)],
-                 "rot": {"dims": 64, "base": 1e6}}
+                 "rot": {"dims": 64, "base": 5e5}}
     q_heads = width // 64
     attention = {"heads": q_heads, "kv_heads": max(1, q_heads // 8), "dim": 64, "vdim": 64,
-                 "scale": 0.125, "softcap": 30.0, "q_temp": {"coef": 0.5, "every": 1024}}
+                 "scale": 0.125, "softcap": 50.0, "q_temp": {"coef": 0.25, "every": 1024}}
     dense = {"kind": "dense", "ff": 4 * width}
     moe = {"kind": "moe", "expert": {"ff": 2 * width}, "router": {"experts": 8, "top": 2}}
     out = []

@@ -71,7 +71,7 @@ TINY_OTHER = config([
     layer("retention", retention(heads=1, dim=32, vdim=32, decay=[0.96875], rot_dims=0), dense(56)),
     layer("retention", retention(heads=4, dim=8, vdim=16, rot_dims=2, base=50.0), None),
     layer("attention", attention(heads=3, kv_heads=3, dim=16, scale=0.45, softcap=9.0, coef=0.1,
-                                 every=64), moe(ff=32, experts=2, top=2)),
+                                 every=50), moe(ff=32, experts=2, top=2)),
 ], width=40, vocab=67, eps=1e-6, logit_scale=1.0)
 
 # a loop that is the whole model and runs once, and one that runs twice from layer 0
@@ -182,14 +182,14 @@ def random_config(seed):
     def rand_retention():
         heads, dim = pick(1, 2, 3, 5), pick(8, 16, 24, 40, 72)
         return retention(heads=heads, dim=dim, vdim=pick(8, 16, 24, 40),
-                         decay=[pick(0.5, 0.9, 0.984375, 0.9990234375, 1.0) for _ in range(heads)],
-                         rot_dims=pick(0, 2, dim // 4 * 2, dim), base=pick(10.0, 1000.0, 1e6))
+                         decay=[pick(0.5, 0.9, 0.96875, 0.99951171875, 1.0) for _ in range(heads)],
+                         rot_dims=pick(0, 2, dim // 4 * 2, dim), base=pick(10.0, 1000.0, 5e5))
 
     def rand_attention():
         kv = pick(1, 2, 3)
         return attention(heads=kv * pick(1, 2, 4), kv_heads=kv, dim=pick(16, 32, 48, 64),
-                         scale=pick(0.1, 0.35, 0.7), softcap=pick(0.0, 1.0, 5.0, 30.0),
-                         coef=pick(-0.2, 0.25, 1.0), every=pick(0, 1, 2, 16, 64))
+                         scale=pick(0.1, 0.35, 0.7), softcap=pick(0.0, 1.0, 5.0, 20.0),
+                         coef=pick(-0.2, 0.25, 1.0), every=pick(0, 1, 2, 16, 48))
 
     def rand_mlp():
         kind = pick("none", "dense", "moe", "moe")
@@ -208,4 +208,4 @@ def random_config(seed):
         start = rng.randrange(n)
         loop = (start, rng.randrange(start + 1, n + 1), pick(1, 2, 3))
     return config(layers, width=pick(16, 24, 40, 64, 104), vocab=pick(11, 50, 203),
-                  eps=pick(1e-6, 1e-5, 1e-3), logit_scale=pick(0.5, 1.0, 2.0), loop=loop)
+                  eps=pick(1e-6, 1e-5, 1e-3), logit_scale=pick(0.5, 1.0, 3.0), loop=loop)

@@ -187,11 +187,11 @@ def test_sink_takes_its_share_and_the_cap_bounds_the_scores():
 
 def test_query_temperature_steps_with_the_position():
     pos = torch.arange(0, 200)
-    f = plain.query_temperature(pos, 0.5, 64)
-    assert float(f[0]) == 1.0 and float(f[62]) == 1.0
-    assert abs(float(f[63]) - (1 + 0.5 * math.log(2))) < 1e-12       # (63 + 1) / 64 = 1
-    assert abs(float(f[127]) - (1 + 0.5 * math.log(3))) < 1e-12
-    assert float(f[126]) == float(f[63])
+    f = plain.query_temperature(pos, 0.25, 40)
+    assert float(f[0]) == 1.0 and float(f[38]) == 1.0
+    assert abs(float(f[39]) - (1 + 0.25 * math.log(2))) < 1e-12      # (39 + 1) / 40 = 1
+    assert abs(float(f[79]) - (1 + 0.25 * math.log(3))) < 1e-12
+    assert float(f[78]) == float(f[39])
 
 
 def test_table_experts_average_their_experts():

@@ -189,7 +189,7 @@ def far_key_model(dtype, dim):
     vector and the last query are made long along one direction, so that the last token's
     output is that key's value if and only if the key is found."""
     cfg = ru.one_layer("attention", ru.attention(heads=2, kv_heads=1, dim=dim, scale=1.0,
-                                                 softcap=50.0, coef=0.2, every=64),
+                                                 softcap=50.0, coef=0.2, every=48),
                        width=64, vocab=300)
     t = ru.make_tensors(cfg, seed=7)
     t["l0.mix.q"] *= 0.05
@@ -243,8 +243,8 @@ def test_the_sink_counts_once_however_the_context_is_cut(dtype):
     # sinks about as large as the logarithm of the keys' summed weights, so that they take
     # about half of every head's weight: left out, counted per range of a cut context, or
     # scaled, they would move every output by tens of percent
-    cfg = ru.one_layer("attention", ru.attention(heads=4, kv_heads=1, dim=64, scale=0.125,
-                                                 softcap=30.0, coef=0.5, every=64),
+    cfg = ru.one_layer("attention", ru.attention(heads=4, kv_heads=1, dim=64, scale=0.11,
+                                                 softcap=25.0, coef=0.4, every=48),
                        width=64, vocab=97)
     tensors = ru.make_tensors(cfg, seed=5)
     n = 1300
@@ -286,7 +286,7 @@ def test_the_query_temperature_changes_where_it_should():
 # ----------------------------------------------------------------- far tokens count
 def test_far_tokens_reach_the_end_through_the_state():
     cfg = ru.one_layer("retention", ru.retention(heads=2, dim=16, vdim=16,
-                                                 decay=[0.9990234375, 1.0], rot_dims=8))
+                                                 decay=[0.99951171875, 1.0], rot_dims=8))
     model, tensors = build(cfg, seed=9)
     n = 600
     a = ru.tokens(n, cfg["vocab"], 3)
@@ -345,13 +345,13 @@ def test_batch_against_each_alone(dtype):
 
 
 # ------------------- sizes that the matrix-core kernels take, at widths of real layers
-@pytest.mark.parametrize("dim,heads,kv", [(64, 8, 1), (128, 4, 2), (64, 16, 4)])
+@pytest.mark.parametrize("dim,heads,kv", [(64, 8, 2), (128, 4, 1), (64, 16, 4)])
 def test_matrix_core_paths(dim, heads, kv):
     cfg = ru.config([
         ru.layer("attention", ru.attention(heads=heads, kv_heads=kv, dim=dim, scale=dim ** -0.5,
-                                           softcap=30.0, coef=0.5, every=64),
+                                           softcap=20.0, coef=0.3, every=50),
                  ru.moe(ff=64, experts=6, top=2)),
-        ru.layer("retention", ru.retention(heads=4, dim=32, vdim=64, rot_dims=32), ru.dense(256)),
+        ru.layer("retention", ru.retention(heads=3, dim=64, vdim=32, rot_dims=16), ru.dense(256)),
     ], width=256, vocab=211, loop=(0, 2, 2))
     model, tensors = build(cfg, seed=6, dtype="bfloat16")
     assert model.blocks[0].parts["mixer"].mfma

@@ -54,7 +54,7 @@ expert_lists_kernel(const int* __restrict__ ids, const int* __restrict__ table, 
     }
     const unsigned long long mask = __ballot(hit);
     const int before = __popcll(mask & ((1ull << lane) - 1ull));
-    __syncthreads();      // the last round's totals have been read
+    __syncthreads();      // the totals of the chunk before have been read
     if (lane == 0) wave_total[wave] = __popcll(mask);
     __syncthreads();
     int offset = running;
@@ -152,7 +152,7 @@ grouped_gemm_bf16_kernel(GroupedArgs g) {
   for (int j = 0; j < NT; ++j) acc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  // steps of 32 a round (two, or four where a wave has one column tile: a decode batch,
+  // steps of 32 at a time (two, or four where a wave has one column tile: a decode batch,
   // which only streams weights): their loads are all requested before the first product
   constexpr int U = NT == 1 ? 4 : 2;
   for (int k0 = 0; k0 < K; k0 += 32 * U) {
