@@ -599,3 +599,19 @@ def test_gated_unit_and_scale_kernels(dtype):
         assert float((out - want).abs().max()) < tol * float(want.abs().max())
     x = torch.randn(5, 9, generator=g)
     assert torch.allclose(ops.scale_(x.to(dev), 2.5).cpu(), x * 2.5)
+
+
+@pytest.mark.parametrize("M,K,I", [(1, 320, 256), (8, 2048, 1024), (16, 512, 136)])
+def test_gate_in_the_product_of_a_decode_batch(M, K, I):
+    """The gate|up product that applies the gate to its own sums, with the tanh form of gelu,
+    against the plain formula on the 32-bit products."""
+    from zig_ai_amd.kernels import ops
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(M + K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(2 * I, K, generator=g) * 2.0 * K ** -0.5).to(torch.bfloat16)
+    for act, fn in (("gelu_tanh", plain.gelu_tanh), ("silu", plain.silu)):
+        got = ops.linear_swiglu(x.to(dev), w.to(dev), act).double().cpu()
+        gu = x.double() @ w.double().T
+        want = fn(gu[:, :I]) * gu[:, I:]
+        assert float((got - want).abs().max()) < 1e-2 * float(want.abs().max()), act

@@ -843,7 +843,8 @@ template <int NW, int KSTEPS, bool NORM, bool STAGED>
 __global__ void __launch_bounds__(NW * 64, 2)
 gemm_bf16_rows16_swiglu_kernel(const bf16_t* __restrict__ A, NormedRowsArg normed,
                                const bf16_t* __restrict__ W, bf16_t* __restrict__ C, int M, int I,
-                               int K, int groups_per_block) {
+                               int K, int groups_per_block, int act) {
+  // `act`: the gate's activation, 0 = silu, 1 = the tanh form of gelu
   __shared__ float red[2][2][NW][64][4];
   __shared__ float ssw[NW][16];
   const int tid = threadIdx.x;
@@ -976,7 +977,10 @@ gemm_bf16_rows16_swiglu_kernel(const bf16_t* __restrict__ A, NormedRowsArg norme
             gv *= scale;
             uv *= scale;
           }
-          C[(size_t)m * I + n] = (bf16_t)(gv * (1.0f / (1.0f + expf(-gv))) * uv);
+          const float gated =
+              act == 1 ? 0.5f * gv * (1.0f + tanhf(0.7978845608028654f * (gv + 0.044715f * gv * gv * gv)))
+                       : gv * (1.0f / (1.0f + expf(-gv)));
+          C[(size_t)m * I + n] = (bf16_t)(gated * uv);
         }
       }
     }
@@ -1229,11 +1233,11 @@ extern "C" int za_gemm_bf16_rows16_merged(const float* part_acc, const float* pa
 // The input is bfloat16 A [M, K], or (A null) rows of the 32-bit stream `x` that the
 // kernel passes through an RMSNorm itself (K <= 4096, K % 512 == 0), as
 // za_gemm_bf16_rows16_stream.
-extern "C" int za_gemm_bf16_rows16_swiglu(const void* A, const float* x, const int* rows,
-                                          const float* norm_weight, float eps, const void* W,
-                                          void* C, int M, int I, int K, hipStream_t stream) {
+static int rows16_gated_any(const void* A, const float* x, const int* rows,
+                            const float* norm_weight, float eps, const void* W, void* C, int M,
+                            int I, int K, int act, hipStream_t stream) {
   if (M == 0 || I == 0) return 0;
-  if (M < 0 || I < 0 || K <= 0 || !W || !C || (!A && !x)) return ZA_ERR_ARG;
+  if (M < 0 || I < 0 || K <= 0 || !W || !C || (!A && !x) || act < 0 || act > 1) return ZA_ERR_ARG;
   if (M > 16 || K % 8 != 0 || K > 8192) return ZA_ERR_UNSUPPORTED;
   const bool norm = !A;
   if (norm && (!norm_weight || !rows16_takes_norm(K, 1))) return ZA_ERR_UNSUPPORTED;
@@ -1250,7 +1254,7 @@ extern "C" int za_gemm_bf16_rows16_swiglu(const void* A, const float* x, const i
     auto kernel = gemm_bf16_rows16_swiglu_kernel<NW, KS, NORM, STAGED>;                       \
     if (const int rc = rows16_allow_lds((const void*)kernel, lds)) return rc;                         \
     hipLaunchKernelGGL(kernel, grid, dim3(NW * 64), lds, stream, (const bf16_t*)A, normed,    \
-                       (const bf16_t*)W, (bf16_t*)C, M, I, K, per_block);                     \
+                       (const bf16_t*)W, (bf16_t*)C, M, I, K, per_block, act);                \
   }
 #define ZA_SG_CASE(NW, KS)                                                                    \
   {                                                                                           \
@@ -1269,6 +1273,20 @@ extern "C" int za_gemm_bf16_rows16_swiglu(const void* A, const float* x, const i
   ZA_SG_CASE(8, 32)
 #undef ZA_SG_CASE
 #undef ZA_SG_LAUNCH
+}
+
+extern "C" int za_gemm_bf16_rows16_swiglu(const void* A, const float* x, const int* rows,
+                                          const float* norm_weight, float eps, const void* W,
+                                          void* C, int M, int I, int K, hipStream_t stream) {
+  return rows16_gated_any(A, x, rows, norm_weight, eps, W, C, M, I, K, 0, stream);
+}
+
+// The same with the gate's activation named: 0 = silu, 1 = the tanh form of gelu.
+extern "C" int za_gemm_bf16_rows16_gated(const void* A, const float* x, const int* rows,
+                                         const float* norm_weight, float eps, const void* W,
+                                         void* C, int M, int I, int K, int act,
+                                         hipStream_t stream) {
+  return rows16_gated_any(A, x, rows, norm_weight, eps, W, C, M, I, K, act, stream);
 }
 
 // The ShortConv mixer from the 32-bit stream to the convolution's output in one kernel

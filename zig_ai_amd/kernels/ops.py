@@ -71,6 +71,9 @@ _SIGNATURES = {
                                              c_int, c_int, c_int, c_void_p],
     ("gemm", "za_gemm_bf16_rows16_swiglu"): [c_void_p, c_void_p, c_void_p, c_void_p, c_float,
                                              c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    ("gemm", "za_gemm_bf16_rows16_gated"): [c_void_p, c_void_p, c_void_p, c_void_p, c_float,
+                                            c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                            c_void_p],
     ("gemm", "za_gemm_bf16_rows16_gated_conv"): [c_void_p, c_void_p, c_void_p, c_float, c_void_p,
                                                  c_void_p, c_void_p, c_void_p, c_longlong,
                                                  c_void_p, c_void_p, c_int, c_int, c_int, c_int,
@@ -797,11 +800,14 @@ def linear(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
     return out
 
 
-def linear_swiglu(x, gate_up_weight: torch.Tensor) -> torch.Tensor:
-    """``silu(x Wg^T) * (x Wu^T)`` for ``gate_up_weight = [Wg; Wu]`` of shape ``[2I, K]``
+def linear_swiglu(x, gate_up_weight: torch.Tensor, activation: str = "silu") -> torch.Tensor:
+    """``act(x Wg^T) * (x Wu^T)`` for ``gate_up_weight = [Wg; Wu]`` of shape ``[2I, K]``
     and at most 16 rows of bfloat16 ``x`` (or a ``NormedRows``): the gate is applied to
     the 32-bit accumulators, the ``[M, 2I]`` intermediate is never stored.  17 to
-    ``ROWS64_SWIGLU_ROWS`` rows are taken as ``NormedRows`` only (``rows64_swiglu_fusable``)."""
+    ``ROWS64_SWIGLU_ROWS`` rows are taken as ``NormedRows`` only (``rows64_swiglu_fusable``),
+    and with ``silu`` only.  ``activation``: one of ``GATE_ACTIVATIONS``."""
+    if activation not in GATE_ACTIVATIONS:
+        raise KernelError(f"activation must be one of {sorted(GATE_ACTIVATIONS)}, got {activation!r}")
     if len(x.shape) != 2 or gate_up_weight.dim() != 2 or gate_up_weight.shape[0] % 2 \
             or gate_up_weight.shape[1] != x.shape[1]:
         raise KernelError(f"linear_swiglu takes x [M, K] and a weight [2I, K], got "
@@ -810,7 +816,7 @@ def linear_swiglu(x, gate_up_weight: torch.Tensor) -> torch.Tensor:
     I = gate_up_weight.shape[0] // 2
     _need(gate_up_weight, "gate_up_weight", torch.bfloat16)
     if M > NORMED_ROWS_MAX_ROWS:
-        if not (isinstance(x, NormedRows) and x.dtype == torch.bfloat16
+        if not (isinstance(x, NormedRows) and x.dtype == torch.bfloat16 and activation == "silu"
                 and rows64_swiglu_fusable(M, K)):
             raise KernelError(f"linear_swiglu takes a step of {M} rows only as rows awaiting "
                               f"their norm, up to {ROWS64_SWIGLU_ROWS} rows, got K={K}")
@@ -829,13 +835,13 @@ def linear_swiglu(x, gate_up_weight: torch.Tensor) -> torch.Tensor:
         raise KernelError(f"linear_swiglu takes at most 16 rows and K <= 8192 in multiples of "
                           f"8, got M={M} K={K}")
     out = torch.empty((M, I), dtype=torch.bfloat16, device=gate_up_weight.device)
-    rc = _fn("gemm", "za_gemm_bf16_rows16_swiglu")(
+    rc = _fn("gemm", "za_gemm_bf16_rows16_gated")(
         None if normed is not None else _ptr(x),
         _ptr(normed.residual) if normed is not None else None,
         _ptr(normed.rows) if normed is not None else None,
         _ptr(normed.weight) if normed is not None else None,
         normed.eps if normed is not None else 0.0,
-        _ptr(gate_up_weight), _ptr(out), M, I, K, _stream())
+        _ptr(gate_up_weight), _ptr(out), M, I, K, GATE_ACTIVATIONS[activation], _stream())
     _check(rc, "linear_swiglu", f"M={M} I={I} K={K}")
     _note("linear_swiglu", M=M, N=2 * I, K=K, norm_in_product=normed is not None)
     return out

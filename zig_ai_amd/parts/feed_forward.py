@@ -57,7 +57,8 @@ class SwiGLU(FeedForward):
         self.gate_up = fuse_rows(tensors["gate.weight"], tensors["up.weight"])
         self.down = tensors["down.weight"]
         # the gate's activation: ``silu`` (SwiGLU) or ``gelu_tanh`` (the tanh form of gelu);
-        # the products that apply the gate to their own sums know silu only
+        # of the products that apply the gate to their own sums the one for decode batches
+        # knows both, the one that also runs the norm of a larger step silu only
         self.activation = str(params.get("activation", "silu"))
         if self.activation not in ops.GATE_ACTIVATIONS:
             raise ValueError(f"feed-forward activation must be one of "
@@ -73,7 +74,13 @@ class SwiGLU(FeedForward):
         if self.activation != "silu":
             if isinstance(x, ops.NormedRows):
                 x = x.materialise()
-            a = ops.gated_unit(ops.linear(x, self.gate_up, tune=self.runtime.tune), self.activation)
+            if x.dtype == torch.bfloat16 and self.gate_up.dtype == torch.bfloat16 \
+                    and x.shape[0] <= 16 and x.shape[1] <= 8192:
+                # a decode batch: the gate is applied to the projection's accumulators
+                a = ops.linear_swiglu(x, self.gate_up, self.activation)
+            else:
+                a = ops.gated_unit(ops.linear(x, self.gate_up, tune=self.runtime.tune),
+                                   self.activation)
             return ops.linear(a, self.down, partial_ok=True, accumulate=stream,
                               tune=self.runtime.tune)
         bf16 = x.dtype == torch.bfloat16 and self.gate_up.dtype == torch.bfloat16
