@@ -615,3 +615,49 @@ def test_gate_in_the_product_of_a_decode_batch(M, K, I):
         gu = x.double() @ w.double().T
         want = fn(gu[:, :I]) * gu[:, I:]
         assert float((got - want).abs().max()) < 1e-2 * float(want.abs().max()), act
+
+
+@pytest.mark.parametrize("H,d,dv", [(2, 16, 8), (3, 64, 128), (1, 128, 40)])
+def test_retention_in_chunks_against_the_plain_walk(H, d, dv):
+    """Long portions walked as chunks side by side: against float64, in two steps so that the
+    second starts from carried states, with portions of exactly one chunk, one more and one
+    fewer, and a decay of one and of a half."""
+    from zig_ai_amd.kernels import ops
+    dev = torch.device("cuda")
+    gen = torch.Generator().manual_seed(d + dv)
+    C = ops.RETENTION_CHUNK
+    steps = [[2 * C + 70, 1, C, C + 1], [C - 1, 3 * C, 5, 1]]
+    decay = torch.tensor(([1.0, 0.5, 0.99609375] * H)[:H])
+    mem, state = _slots(6, 7 + H * d * dv, dev)
+    slots = [4, 0, 5, 2]
+    S64 = [torch.zeros(H, d, dv, dtype=torch.float64) for _ in slots]
+    for lengths in steps:
+        T = sum(lengths)
+        vec = torch.randn(T, 2 * H * d + H * dv, generator=gen)
+        vec[:, H * d:2 * H * d] *= d ** -0.5
+        start, slot_id = _step_arrays(lengths, slots, dev)
+        seq, row0, cnt = [], [], []
+        r = 0
+        for i, n in enumerate(lengths):
+            for a in range(0, n, C):
+                seq.append(i); row0.append(r + a); cnt.append(min(C, n - a))
+            r += n
+        mk = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
+        items = (mk(seq), mk(row0), mk(cnt), len(seq))
+        got = ops.fixed_decay_recurrence_chunked(vec.to(dev), 0, H * d, 2 * H * d, decay.to(dev),
+                                                 state, 7, slot_id, items, H, d, dv).double().cpu()
+        v64 = vec.double()
+        r = 0
+        for i, n in enumerate(lengths):
+            q = v64[r:r + n, :H * d].view(n, H, d)
+            k = v64[r:r + n, H * d:2 * H * d].view(n, H, d)
+            v = v64[r:r + n, 2 * H * d:].view(n, H, dv)
+            for t in range(n):
+                S64[i] = decay.double()[:, None, None] * S64[i] + k[t][:, :, None] * v[t][:, None, :]
+                want = torch.einsum("hdv,hd->hv", S64[i], q[t]).reshape(-1)
+                assert float((got[r + t] - want).abs().max()) < 3e-4 * max(1.0, float(want.abs().max())), (i, t)
+            r += n
+        for i, slot in enumerate(slots):
+            kept = state[slot, 7:].double().cpu().view(H, dv, d).transpose(1, 2)
+            assert float((kept - S64[i]).abs().max()) < 3e-4 * max(1.0, float(S64[i].abs().max()))
+    assert float(mem[:, :7].abs().max()) == 0.0 and float(mem[:, 7 + H * d * dv:].abs().max()) == 0.0

@@ -180,6 +180,8 @@ struct RecurrenceArgs {
   int H, G, dk, dv;
   const float* fixed_decay;   // [H], or null: the SSD walk with this decay, dt = 1 and no
                               // raw step sizes (proj, dt_bias, A_log are not read then)
+  const int* seq_count;       // [n], or null: the walkers' token counts, where their rows
+                              // are given by (start, count) instead of n + 1 starts
 };
 
 // Everything of a token that does not depend on the state, for the delta rule: the unit
@@ -285,7 +287,8 @@ matrix_recurrence_kernel(RecurrenceArgs a) {
   const int g = h / (a.H / a.G);
   const int col = blockIdx.z * (64 / P) + lane / P, part = lane % P;
   const bool owner = col < dv;
-  const int start = a.seq_start[s], n = a.seq_start[s + 1] - start;
+  const int start = a.seq_start[s];
+  const int n = a.seq_count ? a.seq_count[s] : a.seq_start[s + 1] - start;
 
   // where the token's vectors lie: vector v of token t starts at base[v] + t * stride
   const float* base[NV];
@@ -555,7 +558,7 @@ extern "C" int za_matrix_recurrence(int form, int dtype, const float* conv, int 
   RecurrenceArgs a{conv, conv_width, q_col, k_col, x_col, proj, proj_stride, gate_col, dtype,
                    prep, prep_width, dt_bias, A_log, form == 2 ? nullptr : D, state, slot_stride,
                    seq_start, slot_id, out, H, G, dk, dv,
-                   form == 2 ? (const float*)decay : nullptr};
+                   form == 2 ? (const float*)decay : nullptr, nullptr};
   // (a function of the step's shape alone, as a recorded step needs it)
   const bool long_portions = n_tokens > 4 * n_seqs;
   if (form != 1) return launch_recurrence<false>(a, n_seqs, lanes, long_portions, stream);
@@ -573,6 +576,136 @@ extern "C" int za_matrix_recurrence(int form, int dtype, const float* conv, int 
   const int rc = za_launch_status();
   if (rc != 0) return rc;
   return launch_recurrence<true>(a, n_seqs, lanes, long_portions, stream);
+}
+
+// ------------------------------------------------- fixed decay, long portions in chunks
+// With a constant decay a head the state is linear in what the tokens bring, so a long
+// portion need not be walked in one chain.  It is cut into chunks (the step's work items
+// of CHUNK consecutive rows of one request):
+//   1. every chunk is walked by itself from an empty state (matrix_recurrence_kernel with
+//      one walker a chunk), leaving o_local[t] and its own final state L_c;
+//   2. chunk_state_prefix: per request, in the order of its chunks, the state BEFORE chunk c,
+//      B_c = B_(c-1) d^n(c-1) + L_(c-1), B_0 the request's carried state; the last one goes
+//      back to the request's slot.  One thread a state element.
+//   3. chunk_correct: o[t] = o_local[t] + d^(j+1) B_c^T q_t for token j of chunk c.
+// All in 32-bit; powers of the decay as exp2(n log2 d).  A prompt of 2,048 tokens becomes
+// eight chains of 256 tokens side by side instead of one of 2,048.
+__global__ void __launch_bounds__(256)
+chunk_state_prefix_kernel(float* __restrict__ chunk_state, float* __restrict__ state,
+                          long long slot_stride, const int* __restrict__ slot_id,
+                          const int* __restrict__ item_seq, const int* __restrict__ item_count,
+                          int n_items, const float* __restrict__ decay, int elems, int per_head) {
+  const int s = blockIdx.x;
+  const int e = blockIdx.y * 256 + threadIdx.x;
+  if (e >= elems) return;
+  const float l2 = log2f(decay[e / per_head]);
+  float* slot = state + (size_t)slot_id[s] * slot_stride + e;
+  float S = *slot;
+  for (int i = 0; i < n_items; ++i) {
+    if (item_seq[i] != s) continue;
+    float* at = chunk_state + (size_t)i * elems + e;
+    const float local = *at;
+    *at = S;
+    const float a = decay[e / per_head] == 0.f ? 0.f : exp2f((float)item_count[i] * l2);
+    S = fmaf(a, S, local);
+  }
+  *slot = S;
+}
+
+#define CC_TOKENS 16    // tokens whose queries are staged at a time
+template <int DKR>      // rows of a state column kept in registers: dk <= DKR
+__global__ void __launch_bounds__(128)
+chunk_correct_kernel(const float* __restrict__ vectors, int width, int q_col,
+                     const float* __restrict__ chunk_state, const int* __restrict__ item_row0,
+                     const int* __restrict__ item_count, const float* __restrict__ decay,
+                     float* __restrict__ out, int H, int dk, int dv, int tokens_per_block) {
+  __shared__ float qs[CC_TOKENS][DKR];
+  const int item = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int row0 = item_row0[item], cnt = item_count[item];
+  const int t_begin = blockIdx.z * tokens_per_block;
+  int t_end = t_begin + tokens_per_block;
+  if (t_end > cnt) t_end = cnt;
+  if (t_begin >= cnt) return;
+  const float d = decay[h];
+  const float l2 = log2f(d);
+  const size_t elems = (size_t)H * dv * dk;
+  for (int c0 = 0; c0 < dv; c0 += 128) {
+    const int col = c0 + tid;
+    float S[DKR];
+#pragma unroll
+    for (int r = 0; r < DKR; ++r) S[r] = 0.f;
+    if (col < dv) {
+      const float* src = chunk_state + (size_t)item * elems + ((size_t)h * dv + col) * dk;
+#pragma unroll
+      for (int r = 0; r < DKR; ++r)
+        if (r < dk) S[r] = src[r];
+    }
+    for (int tb = t_begin; tb < t_end; tb += CC_TOKENS) {
+      __syncthreads();
+      for (int idx = tid; idx < CC_TOKENS * dk; idx += 128) {
+        const int tt = idx / dk, r = idx % dk;
+        qs[tt][r] = tb + tt < t_end
+                        ? vectors[(size_t)(row0 + tb + tt) * width + q_col + h * dk + r] : 0.f;
+      }
+      __syncthreads();
+      if (col < dv) {
+#pragma unroll 4
+        for (int tt = 0; tt < CC_TOKENS; ++tt) {
+          if (tb + tt >= t_end) break;
+          float dot = 0.f;
+#pragma unroll
+          for (int r = 0; r < DKR; ++r) dot = fmaf(S[r], qs[tt][r], dot);
+          const float w = d == 0.f ? 0.f : exp2f((float)(tb + tt + 1) * l2);
+          float* o = out + (size_t)(row0 + tb + tt) * H * dv + h * dv + col;
+          *o = fmaf(w, dot, *o);
+        }
+      }
+    }
+  }
+}
+
+// `vectors` as retention_prepare leaves them; `item_*`: the step's work items of at most
+// `chunk` rows (n_items of them; with n_items == n_seqs the plain walk does the same); `iota`:
+// 0 .. n_items - 1; `chunk_state`: n_items * H*dv*dk floats, zero on entry.
+extern "C" int za_retention_chunked(const float* vectors, int width, int q_col, int k_col,
+                                    int x_col, const float* decay, float* state,
+                                    long long slot_stride, const int* slot_id,
+                                    const int* item_seq, const int* item_row0,
+                                    const int* item_count, const int* iota, int n_items,
+                                    int n_seqs, int chunk, float* chunk_state, float* out,
+                                    int n_tokens, int H, int dk, int dv, int lanes,
+                                    hipStream_t stream) {
+  if (n_tokens == 0 || n_items == 0) return 0;
+  if (n_tokens < 0 || n_items < n_seqs || n_seqs <= 0 || chunk <= 0 || H <= 0 || dk <= 0 || dv <= 0 ||
+      !vectors || !decay || !state || !slot_id || !item_seq || !item_row0 || !item_count ||
+      !iota || !chunk_state || !out)
+    return ZA_ERR_ARG;
+  if (dk > 128) return ZA_ERR_UNSUPPORTED;
+  if (lanes < 1 || lanes > 64 || (lanes & (lanes - 1)) || lanes * RC_ROWS < dk ||
+      slot_stride < (long long)H * dk * dv)
+    return ZA_ERR_ARG;
+  const long long elems = (long long)H * dk * dv;
+  RecurrenceArgs a{vectors, width, q_col, k_col, x_col, nullptr, 0, 0, 0, nullptr, 0, nullptr,
+                   nullptr, nullptr, chunk_state, elems, item_row0, iota, out, H, H, dk, dv,
+                   decay, item_count};
+  int rc = launch_recurrence<false>(a, n_items, lanes, n_tokens > 4 * n_items, stream);
+  if (rc != 0) return rc;
+  hipLaunchKernelGGL(chunk_state_prefix_kernel, dim3(n_seqs, (unsigned)((elems + 255) / 256)),
+                     dim3(256), 0, stream, chunk_state, state, slot_stride, slot_id, item_seq,
+                     item_count, n_items, decay, (int)elems, dk * dv);
+  rc = za_launch_status();
+  if (rc != 0) return rc;
+  const int tokens_per_block = 64;      // an item has at most `chunk` rows
+  dim3 grid(n_items, H, (unsigned)((chunk + tokens_per_block - 1) / tokens_per_block));
+  if (dk <= 64)
+    hipLaunchKernelGGL((chunk_correct_kernel<64>), grid, dim3(128), 0, stream, vectors, width,
+                       q_col, chunk_state, item_row0, item_count, decay, out, H, dk, dv,
+                       tokens_per_block);
+  else
+    hipLaunchKernelGGL((chunk_correct_kernel<128>), grid, dim3(128), 0, stream, vectors, width,
+                       q_col, chunk_state, item_row0, item_count, decay, out, H, dk, dv,
+                       tokens_per_block);
+  return za_launch_status();
 }
 
 // ------------------------------------------------------------ retention's vectors

@@ -138,6 +138,10 @@ _SIGNATURES = {
         c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
         c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
         c_float, c_void_p, c_float, c_int, c_void_p],
+    ("recurrent", "za_retention_chunked"): [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
+                                            c_longlong, c_void_p, c_void_p, c_void_p, c_void_p,
+                                            c_void_p, c_int, c_int, c_int, c_void_p, c_void_p,
+                                            c_int, c_int, c_int, c_int, c_int, c_void_p],
     ("experts", "za_expert_lists"): [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
                                      c_void_p, c_void_p],
     ("experts", "za_grouped_gemm"): [c_void_p, c_int, c_longlong, c_void_p, c_int, c_void_p,
@@ -1874,6 +1878,49 @@ def _fixed_decay_recurrence(vectors: torch.Tensor, q_col: int, k_col: int, x_col
         0, None, None, None, None, 0, base, slot_stride, _ptr(seq_start), _ptr(slot_id),
         _ptr(out), T, S, heads, groups, dk, dv, lanes, _stream())
     _check(rc, "matrix_recurrence", f"form=fixed heads={heads} dk={dk} dv={dv}")
+    return out
+
+
+RETENTION_CHUNK = 256          # rows of a work item of the chunked fixed-decay walk
+RETENTION_CHUNK_MAX_DK = 128   # state rows the correction keeps in registers
+
+
+def fixed_decay_recurrence_chunked(vectors: torch.Tensor, q_col: int, k_col: int, x_col: int,
+                                   decay: torch.Tensor, state: torch.Tensor, state_offset: int,
+                                   slot_id: torch.Tensor, items, heads: int, dk: int,
+                                   dv: int) -> torch.Tensor:
+    """The fixed-decay walk of ``matrix_recurrence`` for steps with long portions: ``items``
+    (``StepContext.attention_items(RETENTION_CHUNK)``: request, first row, rows, number) cut
+    every request's rows into chunks that are walked side by side from empty states; the
+    states before each chunk follow from a short pass over the chunks, and what they add to
+    each token's read-out is added afterwards (csrc/recurrent.hip).  Same result as the plain
+    walk up to the order of 32-bit additions."""
+    item_seq, item_row0, item_count, n_items = items
+    T, width = vectors.shape
+    S = slot_id.numel()
+    _need(vectors, "vectors", torch.float32)
+    _need(decay, "decay", torch.float32, (heads,))
+    _need(slot_id, "slot_id", torch.int32, (S,))
+    for name, t in (("item_seq", item_seq), ("item_row0", item_row0), ("item_count", item_count)):
+        _need(t, name, torch.int32)
+        if t.numel() < n_items:
+            raise KernelError(f"{name} holds {t.numel()} entries, fewer than {n_items} items")
+    if n_items < S or dk > RETENTION_CHUNK_MAX_DK:
+        raise KernelError(f"{n_items} items for {S} requests, dk={dk}")
+    for name, col, n in (("q_col", q_col, heads * dk), ("k_col", k_col, heads * dk),
+                         ("x_col", x_col, heads * dv)):
+        if col < 0 or col + n > width:
+            raise KernelError(f"{name}: columns {col}..{col + n} of {width}")
+    base, slot_stride = _state_window(state, state_offset, heads * dk * dv, "state")
+    lanes, _, _ = recurrence_plan(dk, dv)
+    out = torch.empty((T, heads * dv), dtype=torch.float32, device=vectors.device)
+    chunk_state = torch.zeros((n_items, heads * dv * dk), dtype=torch.float32, device=vectors.device)
+    iota = torch.arange(n_items, dtype=torch.int32, device=vectors.device)
+    rc = _fn("recurrent", "za_retention_chunked")(
+        _ptr(vectors), width, int(q_col), int(k_col), int(x_col), _ptr(decay), base, slot_stride,
+        _ptr(slot_id), _ptr(item_seq), _ptr(item_row0), _ptr(item_count), _ptr(iota), n_items, S,
+        RETENTION_CHUNK, _ptr(chunk_state), _ptr(out), T, heads, dk, dv, lanes, _stream())
+    _check(rc, "fixed_decay_recurrence_chunked", f"heads={heads} dk={dk} dv={dv} items={n_items}")
     return out
 
 

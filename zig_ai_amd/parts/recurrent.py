@@ -252,6 +252,9 @@ class Retention(Mixer):
         self.w_out = ops.projection_weight(tensors["out_proj.weight"])
         self.gate_col = 2 * H * d + H * dv
         self.ones = torch.ones((1,), dtype=torch.float32, device=runtime.device)
+        # long portions are walked in chunks side by side (the step's work items of that size)
+        self.chunked = d <= ops.RETENTION_CHUNK_MAX_DK
+        self.item_granularities = [ops.RETENTION_CHUNK] if self.chunked else []
         ops.check_projection_weight(self.w_in, "retention opening projection")
         ops.check_projection_weight(self.w_out, "retention out_proj")
 
@@ -262,9 +265,16 @@ class Retention(Mixer):
             z, 0, H * d, 2 * H * d, step.positions,
             self.position.inv_freq if self.rotary_dim else None, H, d, dv, self.rotary_dim,
             self.k_scale)
-        o = ops.matrix_recurrence("fixed", vectors, 0, H * d, 2 * H * d, None, 0, self.decay, None,
-                                  None, None, cache.state, 0, step.seq_start, step.slot_id, H, H,
-                                  d, dv)
+        items = step.attention_items(ops.RETENTION_CHUNK) if self.chunked else None
+        if items is not None and items[3] > step.n_seqs:
+            # some request brings more than a chunk: chunks side by side (a function of the
+            # step's shape alone)
+            o = ops.fixed_decay_recurrence_chunked(vectors, 0, H * d, 2 * H * d, self.decay,
+                                                   cache.state, 0, step.slot_id, items, H, d, dv)
+        else:
+            o = ops.matrix_recurrence("fixed", vectors, 0, H * d, 2 * H * d, None, 0, self.decay,
+                                      None, None, None, cache.state, 0, step.seq_start,
+                                      step.slot_id, H, H, d, dv)
         if getattr(step, "taps", None) is not None:
             step.taps["vectors"] = vectors.clone()
             step.taps["o"] = o.clone()
