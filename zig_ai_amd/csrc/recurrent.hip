@@ -642,22 +642,34 @@ chunk_correct_kernel(const float* __restrict__ vectors, int width, int q_col,
     }
     for (int tb = t_begin; tb < t_end; tb += CC_TOKENS) {
       __syncthreads();
-      for (int idx = tid; idx < CC_TOKENS * dk; idx += 128) {
-        const int tt = idx / dk, r = idx % dk;
-        qs[tt][r] = tb + tt < t_end
+      // (rows beyond dk and tokens beyond the block's end are zeros: every product below
+      // runs over all DKR rows)
+      for (int idx = tid; idx < CC_TOKENS * DKR; idx += 128) {
+        const int tt = idx / DKR, r = idx % DKR;
+        qs[tt][r] = (r < dk && tb + tt < t_end)
                         ? vectors[(size_t)(row0 + tb + tt) * width + q_col + h * dk + r] : 0.f;
       }
       __syncthreads();
       if (col < dv) {
-#pragma unroll 4
-        for (int tt = 0; tt < CC_TOKENS; ++tt) {
-          if (tb + tt >= t_end) break;
-          float dot = 0.f;
+        // what the tokens' read-outs hold is requested for all of them before the first
+        // product, and four sums run side by side in each
+        float* o = out + (size_t)(row0 + tb) * H * dv + h * dv + col;
+        float old[CC_TOKENS];
 #pragma unroll
-          for (int r = 0; r < DKR; ++r) dot = fmaf(S[r], qs[tt][r], dot);
+        for (int tt = 0; tt < CC_TOKENS; ++tt)
+          old[tt] = tb + tt < t_end ? o[(size_t)tt * H * dv] : 0.f;
+#pragma unroll
+        for (int tt = 0; tt < CC_TOKENS; ++tt) {
+          float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
+#pragma unroll
+          for (int r = 0; r < DKR; r += 4) {
+            d0 = fmaf(S[r], qs[tt][r], d0);
+            d1 = fmaf(S[r + 1], qs[tt][r + 1], d1);
+            d2 = fmaf(S[r + 2], qs[tt][r + 2], d2);
+            d3 = fmaf(S[r + 3], qs[tt][r + 3], d3);
+          }
           const float w = d == 0.f ? 0.f : exp2f((float)(tb + tt + 1) * l2);
-          float* o = out + (size_t)(row0 + tb + tt) * H * dv + h * dv + col;
-          *o = fmaf(w, dot, *o);
+          if (tb + tt < t_end) o[(size_t)tt * H * dv] = fmaf(w, (d0 + d1) + (d2 + d3), old[tt]);
         }
       }
     }
