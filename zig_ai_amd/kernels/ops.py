@@ -1795,7 +1795,9 @@ def matrix_recurrence(form: str, conv: torch.Tensor, q_col: int, k_col: int, x_c
                       dt_bias: torch.Tensor, A_log: torch.Tensor, D: Optional[torch.Tensor],
                       state: torch.Tensor, state_offset: int, seq_start: torch.Tensor,
                       slot_id: torch.Tensor, heads: int, groups: int, dk: int, dv: int) -> torch.Tensor:
-    """The token-by-token walk of csrc/recurrent.hip.  ``form``: ``"ssd"`` or ``"delta"``.
+    """The token-by-token walk of csrc/recurrent.hip.  ``form``: ``"ssd"``, ``"delta"`` or
+    ``"fixed"`` (one constant decay a head in ``decay``, 32-bit ``[heads]``; ``proj``, ``dt_bias``,
+    ``A_log`` and ``D`` are not read and may be None: see ``_fixed_decay_recurrence``).
     ``conv [T, columns]`` 32-bit holds, per token, the vectors read against the state's rows
     at ``q_col`` and ``k_col`` (``groups`` of ``dk``) and the one written along its columns at
     ``x_col`` (``heads`` of ``dv``); ``proj [T, columns]`` holds one raw number per head at

@@ -35,6 +35,9 @@ multiplied by ``head_dim^-1/2``; per head ``h``
 then each head's ``o`` over its root mean square (``norm_eps``, no weight), times
 ``silu(g)``, and the output projection.  ``decay`` is a tuple of constants, one a head.
 The state slot holds ``S`` in 32-bit; what enters the walk (rotated q and k, v) is 32-bit.
+A step in which some request brings more than ``ops.RETENTION_CHUNK`` tokens walks its
+portions as chunks side by side (``ops.fixed_decay_recurrence_chunked``): with a constant
+decay the state is linear in what the tokens bring.
 """
 
 from __future__ import annotations
